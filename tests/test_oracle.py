@@ -1,0 +1,374 @@
+"""Pins the CPU oracle (oracle/cvmm_oracle.py) against things the oracle does not define
+itself: library routines (torch.sort, torch.clamp/round, torch.std, einsum), brute-force
+per-token loops, autograd of an independent surrogate, closed forms and invariants.
+Shapes follow the reference's own tests (D=128, E=4, F=64, k=2, 10x10 tokens:
+test_moe_layer_aihwkit_lightning.py:211-217)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cvmm_oracle as O
+
+RNG = np.random.default_rng
+
+
+def _problem(seed=0, T=100, D=128, E=4, F=64, k=2):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, D, generator=g)
+    keys = torch.randn(E, D, F, generator=g) / D ** 0.5
+    values = torch.randn(E, F, D, generator=g) / F ** 0.5
+    router = torch.randn(E, D, generator=g) / D ** 0.5
+    gate, idx = torch.sigmoid(x @ router.t()).topk(k, dim=-1, sorted=False)
+    return x, keys, values, idx, gate
+
+
+# ------------------------------------------------------------------ selection
+@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (33, 4, 1), (512, 8, 2), (4097, 128, 4), (1000, 1000, 8)])
+def test_prepare_sel_matches_stable_sort(M, E, k):
+    M = M - M % k
+    sel = RNG(M).integers(0, E, size=M)
+    s = O.prepare_sel(sel, E, k)
+    ssel, perm = torch.sort(torch.from_numpy(sel), stable=True)
+    assert np.array_equal(s.sel_sorted, ssel.numpy())
+    assert np.array_equal(s.perm, perm.numpy())
+    assert np.array_equal(s.in_index, perm.numpy() // k)
+    assert np.array_equal(np.sort(s.perm), np.arange(M))
+    assert np.array_equal(sel[s.perm], s.sel_sorted)
+    assert s.offsets[0] == 0 and s.offsets[-1] == M
+    for e in range(E):
+        assert np.all(s.sel_sorted[s.offsets[e]:s.offsets[e + 1]] == e)
+
+
+def test_prepare_sel_rejects_bad_ids():
+    with pytest.raises(ValueError):
+        O.prepare_sel(np.array([0, 4]), 4)
+
+
+# ------------------------------------------------------------------ input stage
+def test_kernel_inp_res_mapping():
+    # moe_layer_aihwkit_lightning.py:451-456: both spellings of "8 bit" give 1/127
+    assert O.kernel_inp_res(2 ** 8 - 2) == pytest.approx(1 / 127)
+    assert O.kernel_inp_res(1 / (2 ** 8 - 2)) == pytest.approx(1 / 127)
+    assert O.kernel_inp_res(-1) == -1 and O.kernel_inp_res(0) == -1
+
+
+def test_dac_matches_torch_ops_and_codes_are_8bit():
+    a = (RNG(1).standard_normal((257, 96)) * 2).astype(np.float32)
+    ir = np.abs(RNG(2).standard_normal((257, 1))).astype(np.float32) + 0.3
+    res = np.float32(1 / 127)
+    v, codes = O.dac(a, ir, None, 1 / 127)
+    ta, tir = torch.from_numpy(a), torch.from_numpy(ir)
+    t = torch.clamp(ta, -tir, tir) / tir
+    t = torch.round(t / float(res)) * float(res)
+    assert np.array_equal(v, t.numpy())
+    assert np.array_equal(codes, np.rint(codes)) and np.abs(codes).max() <= 127
+    assert (np.abs(codes) == 127).any()             # some inputs clip at these ranges
+    # quantising an already-quantised, in-range value is the identity
+    v2, _ = O.dac(v * ir, ir, None, 1 / 127)
+    assert np.allclose(v2, v, atol=1e-7)
+
+
+def test_dac_ties_round_to_even():
+    a = np.array([[0.5, 1.5, 2.5, -0.5, -1.5]], dtype=np.float32) / 127
+    v, codes = O.dac(a * np.float32(127) / np.float32(127), None, None, 1 / 127)
+    # 0.5/127/(1/127) is not exactly a tie in fp32, so check rint itself
+    assert np.array_equal(np.rint(np.array([0.5, 1.5, 2.5, -0.5, -1.5], np.float32)), [0, 2, 2, -0, -2])
+    assert np.array_equal(torch.round(torch.tensor([0.5, 1.5, 2.5])).numpy(), [0, 2, 2])
+
+
+def test_dac_off_is_identity():
+    a = RNG(3).standard_normal((5, 7)).astype(np.float32)
+    v, codes = O.dac(a, None, None, -1)
+    assert codes is None and np.array_equal(v, a)
+
+
+# ------------------------------------------------------------------ forward
+def _brute_fwd(x, W, idx, ir=None, res=-1.0):
+    """per-token loop (test_moe_layer_aihwkit_lightning.py:71-80), torch ops only"""
+    T, k = idx.shape
+    out = torch.zeros(T, k, W.shape[2])
+    for t in range(T):
+        for h in range(k):
+            e = int(idx[t, h])
+            a = x[t]
+            if ir is not None:
+                a = torch.clamp(a, -ir[e], ir[e]) / ir[e]
+            if res > 0:
+                a = torch.round(a / res) * res
+            c = a @ W[e]
+            if ir is not None:
+                c = c * ir[e]
+            out[t, h] = c
+    return out
+
+
+def test_fwd_analog_off_is_per_expert_matmul():
+    x, keys, _, idx, _ = _problem()
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    out = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), out_index=s.perm)
+    ref = _brute_fwd(x, keys, idx).reshape(-1, 64).numpy()
+    np.testing.assert_allclose(out, ref, rtol=1e-5, atol=1e-5)
+
+
+def test_fwd_clip_quant_matches_per_token_torch():
+    x, keys, _, idx, _ = _problem(1)
+    ir = torch.tensor([1.0, 2.0, 3.0, 0.5])
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    res = float(np.float32(1 / 127))
+    out, codes = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), 1 / 127,
+                            ir.numpy()[s.sel_sorted], s.perm, return_codes=True)
+    ref = _brute_fwd(x, keys, idx, ir, res).reshape(-1, 64).numpy()
+    np.testing.assert_allclose(out, ref, rtol=1e-5, atol=2e-5)
+    assert np.abs(codes).max() == 127 and np.array_equal(codes, np.rint(codes))
+
+
+def test_fwd_down_projection_layout_and_gate_reduce():
+    x, keys, values, idx, gate = _problem(2)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    p = np.maximum(O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), out_index=s.perm), 0)
+    z = O.cvmm_fwd(p, s.perm, s.sel_sorted, values.numpy())
+    y = O.gate_reduce(z, gate.numpy())
+    # per-token form: test_moe_layer_aihwkit_lightning.py:96-107
+    ref = torch.zeros_like(x)
+    for t in range(x.shape[0]):
+        for h in range(2):
+            e = int(idx[t, h])
+            ref[t] += gate[t, h] * (torch.relu(x[t] @ keys[e]) @ values[e])
+    np.testing.assert_allclose(y, ref.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(y, torch.einsum("tk,tkd->td", gate, torch.from_numpy(z).view(-1, 2, 128)).numpy(),
+                               rtol=1e-5, atol=1e-6)
+
+
+def test_fwd_abs_max_is_scale_equivariant():
+    x, keys, _, idx, _ = _problem(3)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    xn = x.numpy()
+    amax = np.abs(xn).max(-1)
+    f = lambda v, am: O.cvmm_fwd(v, s.in_index, s.sel_sorted, keys.numpy(), 1 / 127, None, s.perm, am)
+    a = f(xn, amax)
+    b = f(4 * xn, 4 * amax)                        # power of two: exact in fp32
+    np.testing.assert_array_equal(4 * a, b)
+    # and it stays within one quantisation step of the un-quantised product
+    ref = _brute_fwd(x, keys, idx).reshape(-1, 64).numpy()
+    assert np.abs(a - ref).max() < 0.05
+
+
+def test_fwd_noise_is_added_before_rescale():
+    x, keys, _, idx, _ = _problem(4)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    ir = np.array([1.0, 2.0, 3.0, 0.5], np.float32)[s.sel_sorted]
+    noise = RNG(5).standard_normal((200, 64)).astype(np.float32) * 0.1
+    args = (x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), 1 / 127, ir, s.perm, None)
+    clean = O.cvmm_fwd(*args)
+    noisy = O.cvmm_fwd(*args, noise)
+    ir_by_out = np.empty(200, np.float32)
+    ir_by_out[s.perm] = ir
+    np.testing.assert_allclose(noisy - clean, noise * ir_by_out[:, None], rtol=0, atol=2e-6)
+
+
+def test_fwd_within_expert_order_does_not_matter():
+    x, keys, _, idx, _ = _problem(5)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    base = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), 1 / 127, None, s.perm,
+                      np.abs(x.numpy()).max(-1))
+    perm2 = s.perm.copy()
+    for e in range(4):
+        seg = slice(s.offsets[e], s.offsets[e + 1])
+        perm2[seg] = perm2[seg][::-1]
+    other = O.cvmm_fwd(x.numpy(), perm2 // 2, s.sel_sorted, keys.numpy(), 1 / 127, None, perm2,
+                       np.abs(x.numpy()).max(-1))
+    np.testing.assert_array_equal(base, other)
+
+
+# ------------------------------------------------------------------ build-defined extensions
+def test_tile_bounds():
+    assert list(O.tile_bounds(1024, 512)) == [0, 512, 1024]
+    assert list(O.tile_bounds(412, 512)) == [0, 412]
+    assert list(O.tile_bounds(412, -1)) == [0, 412]
+    assert list(O.tile_bounds(10, 4)) == [0, 4, 7, 10]
+
+
+def test_tile_split_sums_partials():
+    x, keys, _, idx, _ = _problem(6)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    ir1 = np.full((200, 1), 100.0, np.float32)
+    ir3 = np.full((200, 3), 100.0, np.float32)
+    one = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), -1, ir1, s.perm)
+    three = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), -1, ir3, s.perm,
+                       bounds=O.tile_bounds(128, 48))
+    np.testing.assert_allclose(one, three, rtol=1e-5, atol=1e-5)
+    # with per-tile ranges each tile is its own clip/quantise problem
+    ir_t = np.tile(np.array([[0.5, 1.0, 2.0]], np.float32), (200, 1))
+    split = O.cvmm_fwd(x.numpy(), s.in_index, s.sel_sorted, keys.numpy(), 1 / 127, ir_t, s.perm,
+                       bounds=[0, 43, 86, 128])
+    acc = 0
+    for t, (lo, hi) in enumerate([(0, 43), (43, 86), (86, 128)]):
+        acc = acc + O.cvmm_fwd(x.numpy()[:, lo:hi], s.in_index, s.sel_sorted, keys.numpy()[:, lo:hi], 1 / 127,
+                               ir_t[:, t], s.perm)
+    np.testing.assert_allclose(split, acc, rtol=1e-6, atol=1e-6)
+
+
+def test_adc_off_is_identity_and_on_gives_integer_codes():
+    c = RNG(7).standard_normal((50, 16)).astype(np.float32) * 3
+    wmax = np.full((1, 1), 0.25, np.float32)
+    assert O.adc(c, wmax, -1, -1) is c
+    q = O.adc(c, wmax, 12.0, 2 ** 8 - 2)
+    step = np.float32(12.0 * 0.25 / 127)
+    codes = q / step
+    np.testing.assert_allclose(codes, np.rint(codes), atol=1e-3)
+    assert np.abs(np.rint(codes)).max() <= 127
+    assert np.abs(q - np.clip(c, -3, 3)).max() <= step / 2 + 1e-6
+    clipped_only = O.adc(c * 10, wmax, 12.0, -1)
+    assert np.abs(clipped_only).max() == pytest.approx(3.0)
+
+
+def test_counter_noise_statistics_and_determinism():
+    rows = np.arange(4096)
+    a = O.counter_noise(rows, 256, 0, 1234)
+    assert np.array_equal(a, O.counter_noise(rows, 256, 0, 1234))
+    assert np.array_equal(a[100:200], O.counter_noise(rows[100:200], 256, 0, 1234))
+    b = O.counter_noise(rows, 256, 1, 1234)
+    c = O.counter_noise(rows, 256, 0, 1235)
+    assert abs(a.mean()) < 5e-3 and abs(a.std() - 1) < 5e-3
+    kurt = ((a - a.mean()) ** 4).mean() / a.var() ** 2
+    assert abs(kurt - 3) < 0.05
+    for other in (b, c):
+        assert abs(np.corrcoef(a.ravel(), other.ravel())[0, 1]) < 5e-3
+    assert abs(np.corrcoef(a[:, 0::2].ravel(), a[:, 1::2].ravel())[0, 1]) < 5e-3
+    assert abs(np.corrcoef(a[:-1].ravel(), a[1:].ravel())[0, 1]) < 5e-3
+
+
+# ------------------------------------------------------------------ backward
+def _surrogate_layer(x, keys, values, idx, gate, ir):
+    """Differentiable surrogate with the same straight-through semantics as CVMM.backward:
+    clamp instead of clamp+quantise; per-token loop; autograd supplies every gradient."""
+    T, k = idx.shape
+    y = torch.zeros(T, values.shape[2])
+    zs = torch.zeros(T, k, values.shape[2])
+    for t in range(T):
+        for h in range(k):
+            e = int(idx[t, h])
+            a = x[t] if ir is None else torch.clamp(x[t], -ir[0, e], ir[0, e])
+            p = torch.relu(a @ keys[e])
+            b = p if ir is None else torch.clamp(p, -ir[1, e], ir[1, e])
+            z = b @ values[e]
+            zs[t, h] = z
+            y[t] = y[t] + gate[t, h] * z
+    return y, zs
+
+
+@pytest.mark.parametrize("use_ir", [False, True])
+def test_backward_matches_autograd_of_surrogate(use_ir):
+    x, keys, values, idx, gate = _problem(8, T=60)
+    x.requires_grad_(); keys.requires_grad_(); values.requires_grad_(); gate = gate.detach().requires_grad_()
+    ir = torch.tensor([[1.0, 2.0, 3.0, 4.0], [0.5, 1.0, 1.5, 2.0]]) if use_ir else None
+    y, _ = _surrogate_layer(x, keys, values, idx, gate, ir)
+    dy = torch.randn(y.shape, generator=torch.Generator().manual_seed(1))
+    (y * dy).sum().backward()
+    r = O.layer_fwd_bwd(x.detach().numpy(), keys.detach().numpy(), values.detach().numpy(), idx.numpy(),
+                        gate.detach().numpy(), None if ir is None else ir.numpy()[:, :, None], dy.numpy(),
+                        gradient_relative=False)
+    np.testing.assert_allclose(r.y, y.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_values, values.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_keys, keys.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_x, x.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_gate, gate.grad.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_ir_grad_closed_form_and_special_cases():
+    x, keys, values, idx, gate = _problem(9, T=40)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    g = RNG(1).standard_normal((80, 64)).astype(np.float32)
+    irv = np.array([0.7, 1.0, 1.3, 1.6], np.float32)
+    ir = irv[s.sel_sorted]
+    b = O.cvmm_backward(g, x.numpy(), keys.numpy(), s.sel_sorted, s.in_index, s.perm, None, ir, None, k=2,
+                        gradient_relative=True, gradient_scale=0.5)
+    # brute force, element by element (cvmm.py:848-870)
+    W = keys.numpy().astype(np.float64)
+    want = np.zeros(80)
+    for j in range(80):
+        e, row, o = s.sel_sorted[j], s.in_index[j], s.perm[j]
+        G = g[o].astype(np.float64) @ W[e].T
+        acc = 0.0
+        for n in range(128):
+            xv = x[row, n].item()
+            if xv >= irv[e]:
+                acc += min(G[n], 0.0)
+            if xv <= -irv[e]:
+                acc -= max(G[n], 0.0)
+        want[j] = acc * irv[e] * 0.5
+    np.testing.assert_allclose(b.ir_grad[:, 0], want, rtol=1e-4, atol=1e-5)
+    assert np.abs(want).max() > 0
+    # nothing clips -> zero gradient; decay adds decay*ir when enough inputs are un-clipped
+    big = np.full(80, 100.0, np.float32)
+    b0 = O.cvmm_backward(g, x.numpy(), keys.numpy(), s.sel_sorted, s.in_index, s.perm, None, big, None, k=2)
+    assert np.all(b0.ir_grad == 0)
+    b1 = O.cvmm_backward(g, x.numpy(), keys.numpy(), s.sel_sorted, s.in_index, s.perm, None, big, None, k=2,
+                         decay=0.01, input_min_percentage=0.95)
+    np.testing.assert_allclose(b1.ir_grad[:, 0], 0.01 * big, rtol=1e-6)
+    b2 = O.cvmm_backward(g, x.numpy(), keys.numpy(), s.sel_sorted, s.in_index, s.perm, None, ir, None, k=2,
+                         decay=0.01, input_min_percentage=0.999, gradient_scale=0.5)
+    np.testing.assert_array_equal(b2.ir_grad, b.ir_grad)   # too many inputs clip: no decay term
+
+
+def test_bwd_w_empty_expert_is_zero_and_bf16_rounds():
+    x, keys, _, idx, _ = _problem(10, T=30, E=4)
+    idx = idx.clamp(max=2)                                   # expert 3 gets nothing
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    g = RNG(2).standard_normal((60, 64)).astype(np.float32)
+    gw = O.cvmm_bwd_w(x.numpy(), s.in_index, s.sel_sorted, g, None, 4, s.perm)
+    assert np.all(gw[3] == 0) and np.abs(gw[0]).max() > 0
+    gb = O.cvmm_bwd_w(O.to_bf16(x.numpy()), s.in_index, s.sel_sorted, O.to_bf16(g), None, 4, s.perm, dtype="bf16")
+    assert np.array_equal(gb, O.to_bf16(gb))
+    np.testing.assert_allclose(gb, gw, rtol=3e-2, atol=1e-1)
+
+
+def test_to_bf16_matches_torch():
+    a = RNG(11).standard_normal(10000).astype(np.float32) * 100
+    assert np.array_equal(O.to_bf16(a), torch.from_numpy(a).bfloat16().float().numpy())
+
+
+# ------------------------------------------------------------------ std
+def test_expert_std_matches_torch_std():
+    x, _, _, idx, _ = _problem(12, E=4)
+    idx = idx.clamp(max=2)
+    s = O.prepare_sel(idx.numpy(), 4, 2)
+    got = O.expert_std(x.numpy(), s.in_index, s.sel_sorted, 4)
+    for e in range(3):
+        rows = s.in_index[s.sel_sorted == e]
+        assert got[e] == pytest.approx(torch.std(x[rows].flatten(), unbiased=True).item(), rel=1e-5)
+    assert not (got[3] > 0)                                  # empty expert is filtered by `stds > 0`
+
+
+# ------------------------------------------------------------------ second formulation
+@pytest.mark.parametrize("quant", [False, True])
+def test_per_expert_torch_layer_agrees_with_oracle(quant):
+    from oracle.layer_cpu import moe_layer_per_expert
+    x, keys, values, idx, gate = _problem(13, T=64, E=8, k=2)
+    E = 8
+    ir = torch.tensor(RNG(3).uniform(0.8, 2.5, size=(2, E, 1)).astype(np.float32))
+    wu = keys.abs().amax((1, 2)).reshape(E, 1)
+    wd = values.abs().amax((1, 2)).reshape(E, 1)
+    nu = torch.randn(1, 128, 64, generator=torch.Generator().manual_seed(5)) * 0.04
+    nd = torch.randn(1, 128, 128, generator=torch.Generator().manual_seed(6)) * 0.04
+    nus = nu * wu[idx.reshape(-1)].reshape(1, -1, 1)
+    nds = nd * wd[idx.reshape(-1)].reshape(1, -1, 1)
+    res = 1 / 127 if quant else -1.0
+    ob, orr = (12.0, 254.0) if quant else (-1.0, -1.0)
+    xs = x.clone().requires_grad_(); ks = keys.clone().requires_grad_(); vs = values.clone().requires_grad_()
+    gs = gate.clone().requires_grad_(); irs = ir.clone().requires_grad_()
+    y = moe_layer_per_expert(xs, ks, vs, idx, gs, irs, inp_res=res, noise_up=nus, noise_down=nds,
+                             wmax_up=wu, wmax_down=wd, out_bound=ob, out_res=orr, decay=0.01,
+                             input_min_percentage=0.5)
+    dy = torch.randn(y.shape, generator=torch.Generator().manual_seed(7))
+    (y * dy).sum().backward()
+    r = O.layer_fwd_bwd(x.numpy(), keys.numpy(), values.numpy(), idx.numpy(), gate.numpy(), ir.numpy(), dy.numpy(),
+                        inp_res=res, noise_up=nus.numpy(), noise_down=nds.numpy(), wmax_up=wu.numpy(),
+                        wmax_down=wd.numpy(), out_bound=ob, out_res=orr, decay=0.01, input_min_percentage=0.5)
+    tol = dict(rtol=2e-4, atol=2e-4)
+    np.testing.assert_allclose(r.y, y.detach().numpy(), **tol)
+    np.testing.assert_allclose(r.grad_values, vs.grad.numpy(), **tol)
+    np.testing.assert_allclose(r.grad_keys, ks.grad.numpy(), **tol)
+    np.testing.assert_allclose(r.grad_x, xs.grad.numpy(), **tol)
+    np.testing.assert_allclose(r.grad_gate, gs.grad.numpy(), **tol)
+    np.testing.assert_allclose(r.grad_ir, irs.grad.numpy(), rtol=1e-3, atol=1e-3)
