@@ -1,0 +1,416 @@
+// C ABI of libamoe: argument checks on the host, then kernel launches on the caller's stream.
+#include <amoe.h>
+
+#include "gemm_rows.h"
+#include "gemm_wgrad.h"
+#include "misc_kernels.h"
+#include "prepare_sel.h"
+
+using namespace amoe;
+
+namespace {
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline int launch_rc() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? AMOE_OK : (int)e;
+}
+inline int check_bounds(int n_tiles, const int32_t* b, int K) {
+  if (n_tiles < 1 || n_tiles > AMOE_MAX_TILES) return AMOE_EINVAL;
+  if (b[0] != 0 || b[n_tiles] != K) return AMOE_ESHAPE;
+  for (int t = 0; t < n_tiles; t++)
+    if (b[t + 1] <= b[t]) return AMOE_ESHAPE;
+  return AMOE_OK;
+}
+inline bool bounds_multiple_of(int n_tiles, const int32_t* b, int m) {
+  for (int t = 0; t <= n_tiles; t++)
+    if (b[t] % m) return false;
+  return true;
+}
+inline size_t esize(int dtype) { return dtype == AMOE_F32 ? 4 : 2; }
+inline int max_row_tiles(int64_t M, int E) { return (int)(M / kTileRows) + E; }
+
+template <typename T, bool W_KC>
+int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
+  if (mode == MODE_FWD) {
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD>;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
+  } else if (mode == MODE_FWD_SPLIT) {
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD_SPLIT>;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
+  } else {
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_BWDX>;
+    hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
+  }
+  return launch_rc();
+}
+
+}  // namespace
+
+extern "C" {
+
+int amoe_version(void) { return AMOE_VERSION; }
+
+const char* amoe_strerror(int rc) {
+  switch (rc) {
+    case AMOE_OK: return "ok";
+    case AMOE_EINVAL: return "invalid size, stride or scalar";
+    case AMOE_ENULL: return "required pointer is NULL";
+    case AMOE_ESHAPE: return "inconsistent sizes";
+    case AMOE_EALIGN: return "pointer not aligned to 4 bytes";
+    case AMOE_EWORKSPACE: return "workspace too small";
+    case AMOE_EUNSUPPORTED: return "not supported by this build";
+    default: return rc > 0 ? "HIP launch error" : "unknown error";
+  }
+}
+
+// ------------------------------------------------------------------------------ selection
+size_t amoe_prepare_sel_workspace(int64_t M, int32_t E) {
+  if (M < 0 || E < 1) return 0;
+  const int64_t units = (M + kSelUnit - 1) / kSelUnit;
+  return (size_t)(units > 0 ? units : 1) * (size_t)E * sizeof(int32_t);
+}
+
+int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, int32_t k,
+                     int32_t* sel_sorted, int32_t* perm, int32_t* in_index, int32_t* offsets,
+                     int32_t* bad_flag, void* workspace, size_t workspace_bytes, void* stream) {
+  if (M < 0 || M > 0x7fffffffLL || E < 1 || k < 1) return AMOE_EINVAL;
+  if (E > kSelMaxExperts) return AMOE_EUNSUPPORTED;
+  if (!offsets || !workspace || (M > 0 && (!sel || !sel_sorted || !perm || !in_index))) return AMOE_ENULL;
+  if (!aligned(sel, sel_is_i64 ? 8 : 4) || !aligned(sel_sorted, 4) || !aligned(perm, 4) ||
+      !aligned(in_index, 4) || !aligned(offsets, 4) || !aligned(workspace, 4) || !aligned(bad_flag, 4))
+    return AMOE_EALIGN;
+  if (workspace_bytes < amoe_prepare_sel_workspace(M, E)) return AMOE_EWORKSPACE;
+  SelParams p;
+  p.sel = sel; p.sel_is_i64 = sel_is_i64; p.M = M; p.E = E; p.k = k;
+  p.n_units = (int)((M + kSelUnit - 1) / kSelUnit);
+  p.key_bits = 0;
+  while ((1 << p.key_bits) < E) p.key_bits++;
+  p.sel_sorted = sel_sorted; p.perm = perm; p.in_index = in_index; p.offsets = offsets;
+  p.bad_flag = bad_flag; p.unit_hist = static_cast<int32_t*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int blocks = (p.n_units + 3) / 4;
+  if (blocks > 0) {
+    hipLaunchKernelGGL(sel_hist_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
+    if (int rc = launch_rc()) return rc;
+  }
+  hipLaunchKernelGGL(sel_scan_kernel, dim3(1), dim3(kThreads), 0, st, p);
+  if (int rc = launch_rc()) return rc;
+  if (blocks > 0) {
+    hipLaunchKernelGGL(sel_scatter_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
+    if (int rc = launch_rc()) return rc;
+  }
+  return AMOE_OK;
+}
+
+int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, int32_t* offsets, void* stream) {
+  if (M < 0 || M > 0x7fffffffLL || E < 1) return AMOE_EINVAL;
+  if (!offsets || (M > 0 && !sel_sorted)) return AMOE_ENULL;
+  if (!aligned(sel_sorted, 4) || !aligned(offsets, 4)) return AMOE_EALIGN;
+  const int blocks = (int)((M + 1 + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(blocks), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                     sel_sorted, (long long)M, (int)E, offsets);
+  return launch_rc();
+}
+
+// ------------------------------------------------------------------------------ forward
+int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
+  if (!a) return AMOE_ENULL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->n_in_rows < 0 || a->n_out_rows < 0) return AMOE_EINVAL;
+  if (a->M == 0) return AMOE_OK;
+  if (!a->x || !a->w || !a->out || !a->offsets || !a->in_index) return AMOE_ENULL;
+  if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
+  if (a->ldx < a->K || a->ldo < a->N) return AMOE_ESHAPE;
+  if (a->w_stride_n != 1 && a->w_stride_k != 1) return AMOE_EUNSUPPORTED;
+  const bool gen_noise = a->noise == nullptr && a->noise_std > 0.f;
+  const bool adc = a->out_bound > 0.f;
+  if ((gen_noise || adc) && (!a->wmax || (a->wmax_cols != 1 && a->wmax_cols != a->N))) return AMOE_ESHAPE;
+  if (gen_noise && (a->N % 2)) return AMOE_EUNSUPPORTED;
+  if (a->noise && (a->ldnoise < a->N)) return AMOE_ESHAPE;
+  const size_t es = esize(a->dtype);
+  if (!aligned(a->x, es) || !aligned(a->w, es) || !aligned(a->out, es) || !aligned(a->offsets, 4) ||
+      !aligned(a->in_index, 4) || !aligned(a->out_index, 4) || !aligned(a->ir, 4) || !aligned(a->abs_max, 4) ||
+      !aligned(a->noise, 4) || !aligned(a->wmax, 4) || !aligned(a->range_flag, 4))
+    return AMOE_EALIGN;
+
+  const int CH = a->dtype == AMOE_F32 ? 4 : 8;
+  RowsParams p{};
+  p.M = a->M; p.E = a->E; p.KD = a->K; p.ND = a->N;
+  p.a = a->x; p.lda = a->ldx;
+  p.w = a->w; p.w_se = a->w_stride_e; p.w_skd = a->w_stride_k; p.w_snd = a->w_stride_n;
+  p.out = a->out; p.ldo = a->ldo;
+  p.offsets = a->offsets; p.a_index = a->in_index; p.out_index = a->out_index;
+  p.n_kd_tiles = a->n_tiles;
+  for (int t = 0; t <= a->n_tiles; t++) p.kd_bounds[t] = a->tile_bounds[t];
+  p.n_col_tiles = 1; p.col_bounds[0] = 0; p.col_bounds[1] = a->N;
+  p.n_col_blocks = count_col_blocks(p.col_bounds, 1);
+  p.ir = a->ir; p.ir_cols = a->n_tiles; p.abs_max = a->abs_max; p.inp_res = a->inp_res;
+  p.noise = a->noise; p.noise_ts = a->noise_tile_stride; p.ldnoise = a->ldnoise;
+  p.noise_std = a->noise_std; p.seed = a->noise_seed;
+  p.wmax = a->wmax; p.wmax_cols = a->wmax_cols;
+  p.out_bound = a->out_bound;
+  p.out_half_states = (adc && a->out_res > 0.f) ? 0.5f * fmaxf(a->out_res, 1.0f / a->out_res) : 0.f;
+  p.relu = a->relu; p.range_flag = a->range_flag;
+  const bool w_kc = a->w_stride_n != 1;
+  p.a_vec = aligned(a->x, 16) && (a->ldx % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
+  p.w_vec = aligned(a->w, 16) && (a->w_stride_e % CH == 0) &&
+            (w_kc ? (a->w_stride_n % CH == 0 && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH))
+                  : (a->w_stride_k % CH == 0));
+  p.out_vec = aligned(a->out, 16) && (a->ldo % 4 == 0);
+  p.noise_vec = a->noise && aligned(a->noise, 16) && (a->ldnoise % 4 == 0) && (a->noise_tile_stride % 4 == 0);
+  const int grid = max_row_tiles(a->M, a->E) * p.n_col_blocks;
+  const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a->dtype == AMOE_F32)
+    return w_kc ? launch_rows<float, true>(p, mode, grid, st) : launch_rows<float, false>(p, mode, grid, st);
+  return w_kc ? launch_rows<uint16_t, true>(p, mode, grid, st) : launch_rows<uint16_t, false>(p, mode, grid, st);
+}
+
+// ------------------------------------------------------------------------------ weight gradient
+int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
+  if (!a) return AMOE_ENULL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1) return AMOE_EINVAL;
+  if (!a->grad_w || !a->offsets) return AMOE_ENULL;
+  if (a->M > 0 && (!a->x || !a->g || !a->in_index)) return AMOE_ENULL;
+  if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
+  if (a->M > 0 && (a->ldx < a->K || a->ldg < a->N)) return AMOE_ESHAPE;
+  const size_t es = esize(a->dtype);
+  if (!aligned(a->x, es) || !aligned(a->g, es) || !aligned(a->grad_w, es) || !aligned(a->offsets, 4) ||
+      !aligned(a->in_index, 4) || !aligned(a->g_index, 4) || !aligned(a->ir, 4))
+    return AMOE_EALIGN;
+  const int CH = a->dtype == AMOE_F32 ? 4 : 8;
+  WgradParams p{};
+  p.M = a->M; p.N = a->N; p.K = a->K; p.E = a->E;
+  p.x = a->x; p.ldx = a->ldx; p.g = a->g; p.ldg = a->ldg; p.grad_w = a->grad_w;
+  p.offsets = a->offsets; p.in_index = a->in_index; p.g_index = a->g_index;
+  p.ir = a->ir; p.n_tiles = a->n_tiles;
+  for (int t = 0; t <= a->n_tiles; t++) p.bounds[t] = a->tile_bounds[t];
+  p.n_k_blocks = count_col_blocks(p.bounds, p.n_tiles);
+  p.n_n_blocks = (a->N + kTileCols - 1) / kTileCols;
+  p.x_vec = aligned(a->x, 16) && (a->ldx % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
+  p.g_vec = aligned(a->g, 16) && (a->ldg % CH == 0);
+  p.out_vec = aligned(a->grad_w, 16) && (a->N % 4 == 0);
+  const long long grid = (long long)a->E * p.n_k_blocks * p.n_n_blocks;
+  if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a->dtype == AMOE_F32) {
+    auto k = &gemm_wgrad_kernel<float>;
+    hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
+  } else {
+    auto k = &gemm_wgrad_kernel<uint16_t>;
+    hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
+  }
+  return launch_rc();
+}
+
+// ------------------------------------------------------------------------------ input gradient
+size_t amoe_bwd_x_workspace(int64_t M, int32_t K, int32_t n_tiles) {
+  if (M < 0 || K < 1 || n_tiles < 1) return 0;
+  // worst case: every K-tile adds one partial column block
+  const int64_t col_blocks = (K + kTileCols - 1) / kTileCols + n_tiles;
+  const int64_t row_tiles = M / kTileRows + kSelMaxExperts;
+  return (size_t)(col_blocks * (M > 0 ? M : 1)) * sizeof(float) + (size_t)(row_tiles * col_blocks) * sizeof(int32_t);
+}
+
+int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
+  if (!a) return AMOE_ENULL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->E > kSelMaxExperts) return AMOE_EINVAL;
+  if (a->M == 0) return AMOE_OK;
+  if (!a->g || !a->w || !a->grad_x_full || !a->offsets || !a->g_index || !a->out_index) return AMOE_ENULL;
+  if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
+  const bool use_ir = a->ir != nullptr;
+  if ((use_ir || a->relu_mask) && (!a->x || !a->xf_index)) return AMOE_ENULL;
+  if (use_ir && (!a->ir_grad || !a->workspace)) return AMOE_ENULL;
+  if (a->ldg < a->N || a->ldo < a->K || (a->x && a->ldx < a->K) || a->w_stride_k < a->N) return AMOE_ESHAPE;
+  const size_t es = esize(a->dtype);
+  if (!aligned(a->g, es) || !aligned(a->w, es) || !aligned(a->grad_x_full, es) || !aligned(a->x, es) ||
+      !aligned(a->gate, es) || !aligned(a->offsets, 4) || !aligned(a->g_index, 4) || !aligned(a->out_index, 4) ||
+      !aligned(a->xf_index, 4) || !aligned(a->ir, 4) || !aligned(a->ir_grad, 4) || !aligned(a->workspace, 4))
+    return AMOE_EALIGN;
+  const int CH = a->dtype == AMOE_F32 ? 4 : 8;
+  RowsParams p{};
+  p.M = a->M; p.E = a->E; p.KD = a->N; p.ND = a->K;
+  p.a = a->g; p.lda = a->ldg;
+  p.w = a->w; p.w_se = a->w_stride_e; p.w_skd = 1; p.w_snd = a->w_stride_k;
+  p.out = a->grad_x_full; p.ldo = a->ldo;
+  p.offsets = a->offsets; p.a_index = a->g_index; p.out_index = a->out_index;
+  p.n_kd_tiles = 1; p.kd_bounds[0] = 0; p.kd_bounds[1] = a->N;
+  p.n_col_tiles = a->n_tiles;
+  for (int t = 0; t <= a->n_tiles; t++) p.col_bounds[t] = a->tile_bounds[t];
+  p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles);
+  p.ir = a->ir; p.ir_cols = a->n_tiles; p.inp_res = -1.f;
+  p.xf = a->x; p.ldxf = a->ldx; p.xf_index = a->xf_index; p.gate = a->gate; p.relu_mask = a->relu_mask;
+  const int row_tiles = max_row_tiles(a->M, a->E);
+  const int grid = row_tiles * p.n_col_blocks;
+  if (use_ir) {
+    const size_t need = (size_t)p.n_col_blocks * a->M * sizeof(float) + (size_t)grid * sizeof(int32_t);
+    if (a->workspace_bytes < need) return AMOE_EWORKSPACE;
+    p.irg_partial = static_cast<float*>(a->workspace);
+    p.notclip_count = reinterpret_cast<int32_t*>(p.irg_partial + (size_t)p.n_col_blocks * a->M);
+  }
+  p.a_vec = aligned(a->g, 16) && (a->ldg % CH == 0);
+  p.w_vec = aligned(a->w, 16) && (a->w_stride_e % CH == 0) && (a->w_stride_k % CH == 0);
+  p.out_vec = aligned(a->grad_x_full, 16) && (a->ldo % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
+  p.xf_vec = a->x && aligned(a->x, 16) && (a->ldx % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
+                                : launch_rows<uint16_t, true>(p, MODE_BWDX, grid, st);
+  if (rc) return rc;
+  if (use_ir) {
+    IrFinalizeParams f{};
+    f.M = a->M; f.n_tiles = a->n_tiles; f.KD_total = a->K;
+    for (int t = 0; t <= a->n_tiles; t++) f.col_bounds[t] = a->tile_bounds[t];
+    f.irg_partial = p.irg_partial; f.notclip_count = p.notclip_count; f.n_blocks = grid;
+    f.ir = a->ir; f.ir_grad = a->ir_grad;
+    f.relative = a->gradient_relative; f.scale = a->gradient_scale; f.decay = a->decay;
+    f.min_pct = a->input_min_percentage;
+    hipLaunchKernelGGL(ir_grad_finalize_kernel, dim3((a->M + kThreads - 1) / kThreads), dim3(kThreads), 0, st, f);
+    rc = launch_rc();
+  }
+  return rc;
+}
+
+// ------------------------------------------------------------------------------ row-wise companions
+static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
+                       void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
+  if (T == 0) return AMOE_OK;
+  if (!z || !y) return AMOE_ENULL;
+  const size_t es = esize(dtype);
+  if (!aligned(z, es) || !aligned(y, es) || !aligned(gate, es)) return AMOE_EALIGN;
+  const int vec = aligned(z, 16) && aligned(y, 16) && (D % 4 == 0);
+  const long long work = (long long)T * ((D + 3) / 4);
+  const long long blocks = (work + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &head_reduce_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
+                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D, vec);
+  } else {
+    auto kf = &head_reduce_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
+                       static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D,
+                       vec);
+  }
+  return launch_rc();
+}
+
+int amoe_gate_reduce(int32_t dtype, const void* z, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
+                     void* stream) {
+  if (T > 0 && !gate) return AMOE_ENULL;
+  return head_reduce(dtype, z, gate, y, T, k, D, stream);
+}
+
+int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, int32_t D, void* stream) {
+  return head_reduce(dtype, full, nullptr, out, T, k, D, stream);
+}
+
+int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D,
+                   void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
+  if (T == 0) return AMOE_OK;
+  if (!z || !dy || !grad_gate) return AMOE_ENULL;
+  const size_t es = esize(dtype);
+  if (!aligned(z, es) || !aligned(dy, es) || !aligned(grad_gate, es)) return AMOE_EALIGN;
+  const long long rows = (long long)T * k;
+  const long long blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &gate_grad_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
+                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), rows, (int)k, (int)D);
+  } else {
+    auto kf = &gate_grad_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
+                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), rows, (int)k, (int)D);
+  }
+  return launch_rc();
+}
+
+int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, int32_t K, float* abs_max,
+                     void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (rows < 0 || K < 1 || ldx < K) return AMOE_EINVAL;
+  if (rows == 0) return AMOE_OK;
+  if (!x || !abs_max) return AMOE_ENULL;
+  if (!aligned(x, esize(dtype)) || !aligned(abs_max, 4)) return AMOE_EALIGN;
+  const long long blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &row_abs_max_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(x),
+                       (long long)ldx, (long long)rows, (int)K, abs_max);
+  } else {
+    auto kf = &row_abs_max_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(x),
+                       (long long)ldx, (long long)rows, (int)K, abs_max);
+  }
+  return launch_rc();
+}
+
+int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* wmax,
+                        void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
+  if (!w || !wmax) return AMOE_ENULL;
+  if (!aligned(w, esize(dtype)) || !aligned(wmax, 4)) return AMOE_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (cols == 1 || N == 1) {
+    if (dtype == AMOE_F32) {
+      auto kf = &weight_abs_max_kernel<float>;
+      hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const float*>(w), (long long)K * N, wmax);
+    } else {
+      auto kf = &weight_abs_max_kernel<uint16_t>;
+      hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (long long)K * N, wmax);
+    }
+  } else {
+    dim3 grid((N + kThreads - 1) / kThreads, E);
+    if (dtype == AMOE_F32) {
+      auto kf = &weight_col_abs_max_kernel<float>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, wmax);
+    } else {
+      auto kf = &weight_col_abs_max_kernel<uint16_t>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, wmax);
+    }
+  }
+  return launch_rc();
+}
+
+int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, float* out, void* stream) {
+  if (E < 1 || n_tiles < 1 || n_tiles > AMOE_MAX_TILES) return AMOE_EINVAL;
+  if (!v || !offsets || !out) return AMOE_ENULL;
+  if (!aligned(v, 4) || !aligned(offsets, 4) || !aligned(out, 4)) return AMOE_EALIGN;
+  hipLaunchKernelGGL(segment_sum_kernel, dim3(E, n_tiles), dim3(kThreads), 0, static_cast<hipStream_t>(stream), v,
+                     offsets, (int)n_tiles, out);
+  return launch_rc();
+}
+
+int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K, const int32_t* in_index,
+                    const int32_t* offsets, int32_t E, float* out, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (K < 1 || E < 1 || ldx < K) return AMOE_EINVAL;
+  if (!x || !in_index || !offsets || !out) return AMOE_ENULL;
+  if (!aligned(x, esize(dtype)) || !aligned(in_index, 4) || !aligned(offsets, 4) || !aligned(out, 4))
+    return AMOE_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &expert_std_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const float*>(x), (long long)ldx, (int)K,
+                       in_index, offsets, out);
+  } else {
+    auto kf = &expert_std_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(x), (long long)ldx, (int)K,
+                       in_index, offsets, out);
+  }
+  return launch_rc();
+}
+
+}  // extern "C"

@@ -1,0 +1,239 @@
+// Shared device helpers: element types, bf16 conversion, vector load/store, tile lookup.
+#pragma once
+#include <gfx950_intrin.h>
+#include <stdint.h>
+
+namespace amoe {
+
+constexpr int kThreads = 256;   // 4 waves per workgroup, arranged 2 x 2 over the output tile
+constexpr int kTileRows = 128;  // token rows per workgroup tile
+constexpr int kTileCols = 128;  // feature columns per workgroup tile
+constexpr int kMaxTiles = 16;
+
+// Bit casts through by-value helpers (a bit cast applied directly to a vector element
+// reads element 0 with this compiler).
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// ---- bf16 <-> fp32 (round to nearest even), on raw bits -----------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return as_f32((uint32_t)h << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = as_u32(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// Element traits.  Chunk = 16 bytes of elements, the unit of global and LDS vector access.
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int kChunk = 4;     // elements per 16 bytes
+  static constexpr int kBK = 32;       // contraction elements staged per step (128 B per row)
+  static constexpr int kMmaK = 2;      // contraction elements per matrix instruction
+  static constexpr int kPadKC = 4;     // row padding of the k-contiguous LDS layout
+  static constexpr int kPadRC = 4;     // row padding of the row-contiguous LDS layout
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ float cvt(float v) { return v; }
+  static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+template <> struct Elem<uint16_t> {    // bf16 bits
+  static constexpr int kChunk = 8;
+  static constexpr int kBK = 64;
+  static constexpr int kMmaK = 16;
+  static constexpr int kPadKC = 8;
+  static constexpr int kPadRC = 16;
+  static __device__ __forceinline__ float load(const uint16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ uint16_t cvt(float v) { return f32_to_bf16(v); }
+  static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_to_f32(v); }
+};
+
+// 16 bytes of elements held as fp32 values in registers.
+template <typename T> struct Chunk { float v[Elem<T>::kChunk]; };
+
+template <typename T>
+__device__ __forceinline__ Chunk<T> chunk_zero() {
+  Chunk<T> c;
+#pragma unroll
+  for (int j = 0; j < Elem<T>::kChunk; j++) c.v[j] = 0.f;
+  return c;
+}
+
+// Load one chunk starting at p (elements [0, n_valid) exist; the rest read as zero).
+// vec: p is 16-byte aligned and the caller allows vector access.
+template <typename T>
+__device__ __forceinline__ Chunk<T> chunk_load(const T* p, int n_valid, bool vec) {
+  constexpr int C = Elem<T>::kChunk;
+  Chunk<T> c;
+  if (vec && n_valid >= C) {
+    u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) c.v[j] = as_f32(raw[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        c.v[2 * j] = as_f32(raw[j] << 16);
+        c.v[2 * j + 1] = as_f32(raw[j] & 0xffff0000u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < C; j++) c.v[j] = (j < n_valid) ? Elem<T>::load(p + j) : 0.f;
+  }
+  return c;
+}
+
+// Store one chunk of fp32 values as T into LDS (always 16-byte aligned there).
+template <typename T>
+__device__ __forceinline__ void chunk_store_lds(T* p, const Chunk<T>& c) {
+  u32x4 raw;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) raw[j] = as_u32(c.v[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      raw[j] = (uint32_t)f32_to_bf16(c.v[2 * j]) | ((uint32_t)f32_to_bf16(c.v[2 * j + 1]) << 16);
+  }
+  *reinterpret_cast<u32x4*>(p) = raw;
+}
+
+// Store 4 consecutive fp32 values as T to global memory at p; n_valid of them exist.
+template <typename T>
+__device__ __forceinline__ void store4(T* p, const float (&v)[4], int n_valid, bool vec) {
+  if (vec && n_valid >= 4) {
+    if constexpr (sizeof(T) == 4) {
+      f32x4 o = {v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<f32x4*>(p) = o;
+    } else {
+      u32x2 o;
+      o[0] = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+      o[1] = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+      *reinterpret_cast<u32x2*>(p) = o;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (j < n_valid) p[j] = Elem<T>::cvt(v[j]);
+  }
+}
+
+// Load 4 consecutive elements of T from global memory as fp32.
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float (&v)[4], int n_valid, bool vec) {
+  if (vec && n_valid >= 4) {
+    if constexpr (sizeof(T) == 4) {
+      f32x4 o = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[j] = o[j];
+    } else {
+      u32x2 o = *reinterpret_cast<const u32x2*>(p);
+      v[0] = as_f32(o[0] << 16);
+      v[1] = as_f32(o[0] & 0xffff0000u);
+      v[2] = as_f32(o[1] << 16);
+      v[3] = as_f32(o[1] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = (j < n_valid) ? Elem<T>::load(p + j) : 0.f;
+  }
+}
+
+// ---- row-tile lookup -------------------------------------------------------------------------
+// Sorted positions are cut into tiles of kTileRows rows that never cross an expert boundary.
+// Tile `tile` of the whole list -> (expert, first sorted position, end position).  Every
+// thread of the workgroup calls this; info[0] < 0 means the tile does not exist.
+__device__ __forceinline__ void find_row_tile(const int32_t* __restrict__ offsets, int E, int tile,
+                                              int* info /* LDS int[8] */, int* wave_sums /* LDS int[4] */) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per = (E + kThreads - 1) / kThreads;
+  const int e0 = tid * per;
+  int mine = 0;
+  for (int j = 0; j < per; j++) {
+    int e = e0 + j;
+    if (e < E) mine += (offsets[e + 1] - offsets[e] + kTileRows - 1) / kTileRows;
+  }
+  int incl = mine;  // inclusive scan over the wave
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int up = wave_shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (tid == 0) info[0] = -1;
+  if (lane == 63) wave_sums[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; w++) base += wave_sums[w];
+  int excl = base + incl - mine;
+  if (tile >= excl && tile < excl + mine) {
+    int t = excl;
+    for (int j = 0; j < per; j++) {
+      int e = e0 + j;
+      if (e < E) {
+        int lo = offsets[e], hi = offsets[e + 1];
+        int nt = (hi - lo + kTileRows - 1) / kTileRows;
+        if (tile < t + nt) {
+          int r0 = lo + (tile - t) * kTileRows;
+          info[0] = e;
+          info[1] = r0;
+          info[2] = (r0 + kTileRows < hi) ? r0 + kTileRows : hi;
+          break;
+        }
+        t += nt;
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// Feature blocks of kTileCols columns that restart at every K-tile bound, so that one block
+// lies inside one K-tile.  Block b -> (first column, end column, K-tile).
+struct ColBlock { int c0, c1, tile; };
+__device__ __host__ inline int count_col_blocks(const int32_t* bounds, int n_tiles) {
+  int n = 0;
+  for (int t = 0; t < n_tiles; t++) n += (bounds[t + 1] - bounds[t] + kTileCols - 1) / kTileCols;
+  return n;
+}
+__device__ __forceinline__ ColBlock find_col_block(const int32_t* bounds, int n_tiles, int b) {
+  ColBlock r{0, 0, 0};
+  for (int t = 0; t < n_tiles; t++) {
+    int nb = (bounds[t + 1] - bounds[t] + kTileCols - 1) / kTileCols;
+    if (b < nb) {
+      r.c0 = bounds[t] + b * kTileCols;
+      r.c1 = (r.c0 + kTileCols < bounds[t + 1]) ? r.c0 + kTileCols : bounds[t + 1];
+      r.tile = t;
+      return r;
+    }
+    b -= nb;
+  }
+  return r;
+}
+
+// ---- counter-based Gaussian noise ---------------------------------------------------------------
+// Pure function of (seed, K-tile, output row, column pair): one 32-bit hash per pair, its two
+// 16-bit halves drive one Box-Muller transform.
+__device__ __host__ inline uint32_t fmix32(uint32_t h) {
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  return h;
+}
+struct NoiseKey { uint32_t ka, kb, seed_hi; };
+__device__ __host__ inline NoiseKey noise_key(uint64_t seed, int tile) {
+  NoiseKey k;
+  k.ka = fmix32(((uint32_t)seed ^ 0x9E3779B9u) + (uint32_t)tile * 0x632BE5ABu);
+  k.kb = fmix32(((uint32_t)(seed >> 32) ^ 0x85EBCA77u) + (uint32_t)tile * 0x27D4EB2Fu);
+  k.seed_hi = (uint32_t)(seed >> 32);
+  return k;
+}
+__device__ __forceinline__ void noise_pair(const NoiseKey& key, uint64_t pair_ctr, float& z0, float& z1) {
+  uint32_t h = (uint32_t)pair_ctr ^ key.ka ^ ((uint32_t)(pair_ctr >> 32) * 0xC2B2AE3Du);
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h += key.kb; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  float u1 = ((float)(h >> 16) + 0.5f) * (1.0f / 65536.0f);
+  float u2 = ((float)(h & 0xffffu) + 0.5f) * (1.0f / 65536.0f);
+  float r = fast_sqrt(-2.0f * fast_log(u1));
+  z0 = r * fast_cos_rev(u2);
+  z1 = r * fast_sin_rev(u2);
+}
+
+}  // namespace amoe

@@ -1,0 +1,439 @@
+// Row-gather GEMM of the CVMM path: for every sorted position i of expert e
+//     out[out_index[i], :] = epilogue( prologue(a[a_index[i], :]) @ W[e] )
+// One kernel serves the analog forward (DAC prologue; noise / ADC / rescale epilogue, optional
+// K-tile split) and the input gradient (plain prologue; clip mask, input-range gradient and
+// gate scaling in the epilogue).
+//
+// Workgroup = 256 threads = 2 x 2 waves over a 128 (rows) x 128 (columns) output tile; each
+// wave owns 64 x 64 = 2 x 2 MFMA 32x32 tiles.  The matrix instruction is issued with the
+// weight fragment as its A operand and the token fragment as its B operand, so a lane ends up
+// holding ONE token row (lane % 32) and runs of 4 consecutive output columns: per-row scalars
+// (input range, abs-max, gate, scatter row) are per-lane scalars and stores are 4-wide.
+//
+// LDS layouts:  "KC" [row][k] for operands whose contraction index is contiguous in memory
+// (read with one 16-byte ds_read per fragment), "RC" [k][col] for weights whose output column
+// is contiguous (bf16: read with the transposing ds_read_b64_tr_b16; fp32: plain reads).
+#pragma once
+#include "common.h"
+
+namespace amoe {
+
+enum { MODE_FWD = 0, MODE_FWD_SPLIT = 1, MODE_BWDX = 2 };
+
+struct RowsParams {
+  int M, E;
+  int KD, ND;                       // contraction length, output columns
+  const void* a; int64_t lda;       // gathered operand rows [*, KD]
+  const void* w; int64_t w_se, w_skd, w_snd;  // element strides of W[e][kd][nd]
+  void* out; int64_t ldo;           // [*, ND]
+  const int32_t* offsets; const int32_t* a_index; const int32_t* out_index;
+  int n_kd_tiles; int kd_bounds[kMaxTiles + 1];   // contraction split (forward K-tiles)
+  int n_col_tiles; int col_bounds[kMaxTiles + 1]; // column split (input gradient: K-tiles of x)
+  int n_col_blocks;
+  // forward
+  const float* ir; int ir_cols; const float* abs_max; float inp_res;
+  const float* noise; int64_t noise_ts, ldnoise; float noise_std; uint64_t seed;
+  const float* wmax; int wmax_cols; float out_bound, out_half_states; int relu;
+  int32_t* range_flag;
+  // input gradient
+  const void* xf; int64_t ldxf; const int32_t* xf_index; const void* gate;
+  float* irg_partial; int32_t* notclip_count; int relu_mask;
+  // vector-access permissions (alignment checked on the host)
+  int a_vec, w_vec, out_vec, noise_vec, xf_vec;
+};
+
+template <typename T, bool W_KC, int MODE>
+__global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p) {
+  using EL = Elem<T>;
+  constexpr int BK = EL::kBK, CH = EL::kChunk, MMAK = EL::kMmaK;
+  constexpr int LDA = BK + EL::kPadKC;
+  constexpr int LDB = W_KC ? (BK + EL::kPadKC) : (kTileCols + EL::kPadRC);
+  constexpr int B_ELEMS = W_KC ? kTileCols * LDB : BK * LDB;
+  constexpr bool IS_BF16 = sizeof(T) == 2;
+  constexpr bool FWD = MODE != MODE_BWDX;
+
+  __shared__ __attribute__((aligned(16))) T sA[kTileRows * LDA];
+  __shared__ __attribute__((aligned(16))) T sB[B_ELEMS];
+  __shared__ __attribute__((aligned(16))) float sCol[4][kTileCols];
+  __shared__ float sRed[2][kTileRows];
+  __shared__ int sCnt[4];
+  __shared__ int sInfo[8];
+  __shared__ int sWave[4];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const int row_tile = blockIdx.x / p.n_col_blocks;
+  const int cb = blockIdx.x % p.n_col_blocks;
+  find_row_tile(p.offsets, p.E, row_tile, sInfo, sWave);
+  const int e = sInfo[0];
+  if (e < 0) {
+    if (MODE == MODE_BWDX && tid == 0 && p.notclip_count) p.notclip_count[blockIdx.x] = 0;
+    return;
+  }
+  const int row0 = sInfo[1], row_end = sInfo[2];
+  const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb);
+  const int c0 = colb.c0, c1 = colb.c1;
+
+  const T* __restrict__ A = static_cast<const T*>(p.a);
+  const T* __restrict__ W = static_cast<const T*>(p.w) + (int64_t)e * p.w_se;
+  T* __restrict__ OUT = static_cast<T*>(p.out);
+
+  const bool has_ir = FWD && p.ir != nullptr;
+  const bool has_amax = FWD && p.abs_max != nullptr;
+  const bool quant = FWD && p.inp_res > 0.f;
+  const bool codes_mode = IS_BF16 && quant;   // feed integer codes, scale the accumulator
+  const bool adc_clip = FWD && p.out_bound > 0.f;
+  const bool adc_quant = adc_clip && p.out_half_states > 0.f;
+  const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
+
+  // ---- per-column constants of the forward epilogue --------------------------------------
+  if (FWD && tid < kTileCols) {
+    const int col = c0 + tid;
+    float wm = 1.f;
+    if (p.wmax != nullptr && col < c1) wm = p.wmax[(int64_t)e * p.wmax_cols + (p.wmax_cols > 1 ? col : 0)];
+    const float bound = p.out_bound * wm;
+    sCol[0][tid] = p.noise_std * wm;
+    sCol[1][tid] = bound;
+    sCol[2][tid] = adc_quant ? p.out_half_states / bound : 0.f;
+    sCol[3][tid] = adc_quant ? bound / p.out_half_states : 0.f;
+  }
+
+  // ---- staging assignments ------------------------------------------------------------------
+  // A (and KC weights): thread -> rows tid/8 + 32*i (i < 4), 16-byte chunk tid%8 of the step.
+  const int a_chunk = tid & 7;
+  const T* a_row[4];
+  bool a_ok[4];
+  float a_amax[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = row0 + (tid >> 3) + 32 * i;
+    a_ok[i] = r < row_end;
+    const int idx = a_ok[i] ? p.a_index[r] : 0;
+    a_row[i] = A + (int64_t)idx * p.lda;
+    a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[idx] : 1.f;
+  }
+  // RC weights: thread -> contraction rows tid/CPR + RPP*i, chunk tid%CPR of the 128 columns.
+  constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
+  static_assert(BK == 4 * RPP, "RC staging expects 4 passes");
+
+  f32x16 acc[2][2];
+  f32x16 total[2][2];
+  if (MODE == MODE_FWD_SPLIT) {
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+      for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) total[a][b][i] = 0.f;
+  }
+
+  for (int t = 0; t < p.n_kd_tiles; t++) {
+    const int klo = p.kd_bounds[t], khi = p.kd_bounds[t + 1];
+    const int nsteps = (khi - klo + BK - 1) / BK;
+    float a_ir[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int r = row0 + (tid >> 3) + 32 * i;
+      a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)r * p.ir_cols + t] : 1.f;
+    }
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+      for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+
+    Chunk<T> ra[4], rb[4];
+    auto load_step = [&](int s) {
+      const int k0 = klo + s * BK;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int kpos = k0 + a_chunk * CH;
+        int nv = a_ok[i] ? khi - kpos : 0;
+        nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
+        ra[i] = chunk_load<T>(a_row[i] + kpos, nv, p.a_vec != 0);
+      }
+      if (W_KC) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int col = c0 + (tid >> 3) + 32 * i;
+          const int kpos = k0 + a_chunk * CH;
+          int nv = col < c1 ? khi - kpos : 0;
+          nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
+          rb[i] = chunk_load<T>(W + (int64_t)col * p.w_snd + kpos, nv, p.w_vec != 0);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int kd = k0 + tid / CPR + RPP * i;
+          const int col = c0 + (tid % CPR) * CH;
+          int nv = kd < khi ? c1 - col : 0;
+          nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
+          rb[i] = chunk_load<T>(W + (int64_t)kd * p.w_skd + col, nv, p.w_vec != 0);
+        }
+      }
+    };
+
+    load_step(0);
+    for (int s = 0; s < nsteps; s++) {
+      // ---- prologue on the gathered rows, then registers -> LDS ------------------------------
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        if (FWD && (has_ir || has_amax || quant)) {
+          bool out_of_range = false;
+#pragma unroll
+          for (int j = 0; j < CH; j++) {
+            float v = ra[i].v[j];
+            if (has_ir) {
+              const float r = a_ir[i];
+              v = v > r ? r : v;
+              v = v < -r ? -r : v;
+              v = v / r;
+            }
+            if (has_amax) v = v / a_amax[i];
+            if (quant) {
+              out_of_range |= !(fabsf(v) <= 1.0f);
+              v = rintf(v / p.inp_res);
+              if (!IS_BF16) v = v * p.inp_res;
+            }
+            ra[i].v[j] = v;
+          }
+          if (quant && out_of_range && a_ok[i] && p.range_flag != nullptr) atomicOr(p.range_flag, 1);
+        }
+        chunk_store_lds<T>(&sA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH], ra[i]);
+        if (W_KC) chunk_store_lds<T>(&sB[((tid >> 3) + 32 * i) * LDB + a_chunk * CH], rb[i]);
+        else chunk_store_lds<T>(&sB[(tid / CPR + RPP * i) * LDB + (tid % CPR) * CH], rb[i]);
+      }
+      __syncthreads();
+      if (s + 1 < nsteps) load_step(s + 1);
+
+      // ---- matrix instructions -----------------------------------------------------------------
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += MMAK) {
+        if constexpr (IS_BF16) {
+          u32x4 xf[2], wf[2];
+#pragma unroll
+          for (int ti = 0; ti < 2; ti++)
+            xf[ti] = *reinterpret_cast<const u32x4*>(&sA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++) {
+            if (W_KC) {
+              wf[fi] = *reinterpret_cast<const u32x4*>(&sB[(wc * 64 + fi * 32 + l32) * LDB + kk + 8 * lh]);
+            } else {
+              const int R = lane & 15, g = (lane >> 4) & 1;
+              const uint16_t* base = reinterpret_cast<const uint16_t*>(
+                  &sB[(kk + 8 * lh + (R >> 2)) * LDB + wc * 64 + fi * 32 + 16 * g + 4 * (R & 3)]);
+              u32x2 lo = lds_read_tr16_b64(base);
+              u32x2 hi = lds_read_tr16_b64(base + 4 * LDB);
+              wf[fi] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+          }
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
+        } else {
+          float xf[2], wf[2];
+#pragma unroll
+          for (int ti = 0; ti < 2; ti++) xf[ti] = sA[(wr * 64 + ti * 32 + l32) * LDA + kk + lh];
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++)
+            wf[fi] = W_KC ? sB[(wc * 64 + fi * 32 + l32) * LDB + kk + lh]
+                          : sB[(kk + lh) * LDB + wc * 64 + fi * 32 + l32];
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x2_f32(wf[fi], xf[ti], acc[fi][ti]);
+        }
+      }
+      __syncthreads();
+    }
+
+    // ---- per-K-tile analog output stage (forward) ------------------------------------------------
+    if (FWD) {
+      const NoiseKey key = noise_key(p.seed, t);
+#pragma unroll
+      for (int ti = 0; ti < 2; ti++) {
+        const int r = row0 + wr * 64 + ti * 32 + l32;
+        const bool valid = r < row_end;
+        const int arow = valid ? p.a_index[r] : 0;
+        const int orow = valid ? (p.out_index ? p.out_index[r] : arow) : 0;
+        const float ir_r = (has_ir && valid) ? p.ir[(int64_t)r * p.ir_cols + t] : 1.f;
+        const float am_r = (has_amax && valid) ? p.abs_max[arow] : 1.f;
+#pragma unroll
+        for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const int cl = wc * 64 + fi * 32 + 8 * q + 4 * lh;
+            const int col = c0 + cl;
+            int nv = valid ? c1 - col : 0;
+            nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
+            if (codes_mode) {
+#pragma unroll
+              for (int j = 0; j < 4; j++) v[j] *= p.inp_res;
+            }
+            if (p.noise != nullptr) {
+              float nz[4];
+              load4<float>(p.noise + (int64_t)t * p.noise_ts + (int64_t)orow * p.ldnoise + col, nz, nv,
+                           p.noise_vec != 0);
+#pragma unroll
+              for (int j = 0; j < 4; j++) v[j] += nz[j];
+            } else if (gen_noise) {
+              float z[4];
+              const uint64_t ctr = (uint64_t)orow * (uint64_t)(p.ND >> 1) + (uint64_t)(col >> 1);
+              noise_pair(key, ctr, z[0], z[1]);
+              noise_pair(key, ctr + 1, z[2], z[3]);
+#pragma unroll
+              for (int j = 0; j < 4; j++) v[j] += sCol[0][cl + j] * z[j];
+            }
+            if (adc_clip) {
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                const float b = sCol[1][cl + j];
+                v[j] = fminf(fmaxf(v[j], -b), b);
+                if (adc_quant) v[j] = rintf(v[j] * sCol[2][cl + j]) * sCol[3][cl + j];
+              }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              if (has_amax) v[j] *= am_r;
+              if (has_ir) v[j] *= ir_r;
+              if (MODE == MODE_FWD_SPLIT) total[fi][ti][4 * q + j] += v[j];
+              else acc[fi][ti][4 * q + j] = v[j];
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- store ---------------------------------------------------------------------------------------
+  if (FWD) {
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++) {
+      const int r = row0 + wr * 64 + ti * 32 + l32;
+      const bool valid = r < row_end;
+      const int orow = valid ? (p.out_index ? p.out_index[r] : p.a_index[r]) : 0;
+#pragma unroll
+      for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
+          int nv = valid ? c1 - col : 0;
+          nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            v[j] = (MODE == MODE_FWD_SPLIT) ? total[fi][ti][4 * q + j] : acc[fi][ti][4 * q + j];
+            if (p.relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
+          }
+          if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
+        }
+      }
+    }
+  } else {
+    // ---- input gradient: clip mask, input-range gradient partial sums, gate ---------------------
+    const T* __restrict__ XF = static_cast<const T*>(p.xf);
+    const T* __restrict__ GATE = static_cast<const T*>(p.gate);
+    const bool use_ir = p.ir != nullptr;
+    int cnt = 0;
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++) {
+      const int rl = wr * 64 + ti * 32 + l32;
+      const int r = row0 + rl;
+      const bool valid = r < row_end;
+      const int orow = valid ? p.out_index[r] : 0;
+      const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
+      const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
+      const float ir_r = (use_ir && valid) ? p.ir[(int64_t)r * p.ir_cols + colb.tile] : 0.f;
+      float part = 0.f;
+#pragma unroll
+      for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
+          int nv = valid ? c1 - col : 0;
+          nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+          float v[4], xv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, p.xf_vec != 0);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            float g = acc[fi][ti][4 * q + j];
+            if (j < nv) {
+              if (use_ir) {
+                const float gs = g * gate_r;
+                if (xv[j] >= ir_r) part += fminf(gs, 0.f);
+                if (xv[j] <= -ir_r) part -= fmaxf(gs, 0.f);
+                const bool not_clip = fabsf(xv[j]) < ir_r;
+                cnt += not_clip ? 1 : 0;
+                g = not_clip ? g : 0.f;
+              }
+              if (p.relu_mask) g = xv[j] > 0.f ? g : 0.f;
+            }
+            v[j] = g * gate_r;
+          }
+          if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
+        }
+      }
+      if (use_ir) {
+        part += wave_shfl_xor(part, 32);
+        if (lh == 0) sRed[wc][rl] = part;
+      }
+    }
+    if (use_ir) {
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) cnt += wave_shfl_xor(cnt, d);
+      if (lane == 0) sCnt[wave] = cnt;
+      __syncthreads();
+      if (tid < kTileRows && row0 + tid < row_end)
+        p.irg_partial[(int64_t)cb * p.M + row0 + tid] = sRed[0][tid] + sRed[1][tid];
+      if (tid == 0) p.notclip_count[blockIdx.x] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
+    }
+  }
+}
+
+// Sum the column-block partials into ir_grad[M, n_tiles] and apply the scaling and decay rules.
+struct IrFinalizeParams {
+  int M, n_tiles, KD_total;      // KD_total = columns of x (for the un-clipped fraction)
+  int col_bounds[kMaxTiles + 1];
+  const float* irg_partial; const int32_t* notclip_count; int n_blocks;
+  const float* ir; float* ir_grad;
+  int relative; float scale, decay, min_pct;
+};
+
+__global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFinalizeParams p) {
+  __shared__ long long sTot[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float flag = 0.f;
+  if (p.decay > 0.f) {
+    long long c = 0;
+    for (int i = tid; i < p.n_blocks; i += kThreads) c += p.notclip_count[i];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) c += wave_shfl_xor(c, d);
+    if (lane == 0) sTot[wave] = c;
+    __syncthreads();
+    const long long tot = sTot[0] + sTot[1] + sTot[2] + sTot[3];
+    const float pct = (float)tot / (float)((long long)p.M * (long long)p.KD_total);
+    flag = pct > p.min_pct ? 1.f : 0.f;
+  }
+  const int r = blockIdx.x * kThreads + tid;
+  if (r >= p.M) return;
+  int cb = 0;
+  for (int t = 0; t < p.n_tiles; t++) {
+    const int nb = (p.col_bounds[t + 1] - p.col_bounds[t] + kTileCols - 1) / kTileCols;
+    float s = 0.f;
+    for (int b = 0; b < nb; b++) s += p.irg_partial[(int64_t)(cb + b) * p.M + r];
+    cb += nb;
+    const float irv = p.ir[(int64_t)r * p.n_tiles + t];
+    if (p.relative) s = s * irv * p.scale;
+    if (p.decay > 0.f) s = s + p.decay * irv * flag;
+    p.ir_grad[(int64_t)r * p.n_tiles + t] = s;
+  }
+}
+
+}  // namespace amoe

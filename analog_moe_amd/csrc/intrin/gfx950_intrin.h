@@ -1,0 +1,65 @@
+// gfx950 (CDNA4) instruction wrappers used by the CVMM kernels.
+//
+// Operand layouts of the two matrix instructions used here, for lane l of a 64-wide wave
+// (measured on MI355X with one-hot operands):
+//   v_mfma_f32_32x32x16_bf16: A lane l holds A[l%32][8*(l/32) .. +7], B lane l holds
+//     B[8*(l/32) .. +7][l%32]; D lane l holds D[8*(i/4) + 4*(l/32) + i%4][l%32], i = 0..15.
+//   v_mfma_f32_32x32x2_f32:   A lane l holds A[l%32][l/32], B lane l holds B[l/32][l%32];
+//     D as above.
+//   ds_read_b64_tr_b16: within each group of 16 lanes, lane R supplies the address of four
+//     consecutive 16-bit elements (a "row"); lane i receives element (i%4) of rows
+//     i/4, i/4+4, i/4+8, i/4+12.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace amoe {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+
+__device__ __forceinline__ f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// Transposing 64-bit LDS read of 16-bit elements; p is this lane's row address in LDS.
+__device__ __forceinline__ u32x2 lds_read_tr16_b64(const uint16_t* p) {
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (s16x4 __attribute__((address_space(3)))*)(p));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+template <typename V>
+__device__ __forceinline__ V wave_shfl_xor(V v, int mask) { return __shfl_xor(v, mask, 64); }
+template <typename V>
+__device__ __forceinline__ V wave_shfl(V v, int src) { return __shfl(v, src, 64); }
+template <typename V>
+__device__ __forceinline__ V wave_shfl_up(V v, int d) { return __shfl_up(v, d, 64); }
+__device__ __forceinline__ uint64_t wave_ballot(bool p) { return __ballot(p); }
+__device__ __forceinline__ int popc64(uint64_t v) { return __popcll(v); }
+// Orders this wave's LDS accesses before the barrier against those after it.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// sin / cos of 2*pi*x (x in revolutions), natural log, sqrt: single hardware instructions.
+__device__ __forceinline__ float fast_sin_rev(float x) { return __builtin_amdgcn_sinf(x); }
+__device__ __forceinline__ float fast_cos_rev(float x) { return __builtin_amdgcn_cosf(x); }
+__device__ __forceinline__ float fast_log(float x) { return __logf(x); }
+__device__ __forceinline__ float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ uint32_t umulhi32(uint32_t a, uint32_t b) { return __umulhi(a, b); }
+
+}  // namespace amoe

@@ -1,0 +1,141 @@
+// Row-wise companions of the CVMM calls: gate-weighted reduction over the k heads, k-sum,
+// gate gradient, abs-max of rows and of weights, per-expert segment sums and standard
+// deviation.  All are bandwidth-bound streaming kernels with fixed summation order.
+#pragma once
+#include "common.h"
+
+namespace amoe {
+
+// y[t, d] = sum_j gate[t*k+j] * z[(t*k+j), d]   (gate == nullptr: plain sum over j)
+template <typename T>
+__global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restrict__ z, const T* __restrict__ gate,
+                                                                T* __restrict__ y, long long rows, int k, int D,
+                                                                int vec) {
+  const int quads = (D + 3) / 4;
+  const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+  if (idx >= rows * quads) return;
+  const long long t = idx / quads;
+  const int d = (int)(idx % quads) * 4;
+  const int nv = D - d < 4 ? D - d : 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < k; j++) {
+    float v[4];
+    load4<T>(z + (t * k + j) * (long long)D + d, v, nv, vec != 0);
+    const float gt = gate ? Elem<T>::load(gate + t * k + j) : 1.f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) acc[q] += gt * v[q];
+  }
+  store4<T>(y + t * (long long)D + d, acc, nv, vec != 0);
+}
+
+// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>, one wave per row.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict__ z, const T* __restrict__ dy,
+                                                              T* __restrict__ out, long long rows, int k, int D) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  float s = 0.f;
+  if (row < rows) {
+    const T* zr = z + row * (long long)D;
+    const T* dr = dy + (row / k) * (long long)D;
+    for (int d = lane; d < D; d += 64) s += Elem<T>::load(zr + d) * Elem<T>::load(dr + d);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
+  if (row < rows && lane == 0) out[row] = Elem<T>::cvt(s);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void row_abs_max_kernel(const T* __restrict__ x, long long ldx, long long rows,
+                                                                int K, float* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  float m = 0.f;
+  if (row < rows)
+    for (int d = lane; d < K; d += 64) m = fmaxf(m, fabsf(Elem<T>::load(x + row * ldx + d)));
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, wave_shfl_xor(m, d));
+  if (row < rows && lane == 0) out[row] = m;
+}
+
+// cols == N: wmax[e, c] = max_k |w[e, k, c]|, one thread per column.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void weight_col_abs_max_kernel(const T* __restrict__ w, int K, int N,
+                                                                       float* __restrict__ out) {
+  const int e = blockIdx.y;
+  const int c = blockIdx.x * kThreads + threadIdx.x;
+  if (c >= N) return;
+  const T* base = w + (long long)e * K * N + c;
+  float m = 0.f;
+  for (int k = 0; k < K; k++) m = fmaxf(m, fabsf(Elem<T>::load(base + (long long)k * N)));
+  out[(long long)e * N + c] = m;
+}
+// cols == 1: wmax[e] = max |w[e]|, one workgroup per expert.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __restrict__ w, long long per_expert,
+                                                                   float* __restrict__ out) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const T* base = w + (long long)blockIdx.x * per_expert;
+  float m = 0.f;
+  for (long long i = tid; i < per_expert; i += kThreads) m = fmaxf(m, fabsf(Elem<T>::load(base + i)));
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, wave_shfl_xor(m, d));
+  if (lane == 0) red[tid >> 6] = m;
+  __syncthreads();
+  if (tid == 0) out[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// out[e, t] = sum_{i in [offsets[e], offsets[e+1])} v[i, t], one workgroup per (expert, tile).
+__global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float* __restrict__ v,
+                                                                const int32_t* __restrict__ offsets, int n_tiles,
+                                                                float* __restrict__ out) {
+  __shared__ float red[4];
+  const int e = blockIdx.x, t = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63;
+  float s = 0.f;
+  for (int i = offsets[e] + tid; i < offsets[e + 1]; i += kThreads) s += v[(long long)i * n_tiles + t];
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
+  if (lane == 0) red[tid >> 6] = s;
+  __syncthreads();
+  if (tid == 0) out[(long long)e * n_tiles + t] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__device__ __forceinline__ double block_sum_double(double v, double* red /* LDS [4] */) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += wave_shfl_xor(v, d);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// Two-pass unbiased std over all elements of the rows of one expert (one workgroup per expert).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void expert_std_kernel(const T* __restrict__ x, long long ldx, int K,
+                                                               const int32_t* __restrict__ in_index,
+                                                               const int32_t* __restrict__ offsets,
+                                                               float* __restrict__ out) {
+  __shared__ double red[4];
+  const int e = blockIdx.x, tid = threadIdx.x;
+  const int lo = offsets[e], hi = offsets[e + 1];
+  const long long n = (long long)(hi - lo) * K;
+  double s = 0.0;
+  for (long long i = tid; i < n; i += kThreads) {
+    const int r = lo + (int)(i / K), c = (int)(i % K);
+    s += (double)Elem<T>::load(x + (long long)in_index[r] * ldx + c);
+  }
+  s = block_sum_double(s, red);
+  const double mean = n > 0 ? s / (double)n : 0.0;
+  double ss = 0.0;
+  for (long long i = tid; i < n; i += kThreads) {
+    const int r = lo + (int)(i / K), c = (int)(i % K);
+    const double d = (double)Elem<T>::load(x + (long long)in_index[r] * ldx + c) - mean;
+    ss += d * d;
+  }
+  ss = block_sum_double(ss, red);
+  if (tid == 0) out[e] = (n == 0) ? -0.0f : (float)sqrt(ss / (double)(n - 1));
+}
+
+}  // namespace amoe

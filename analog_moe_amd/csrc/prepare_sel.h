@@ -1,0 +1,146 @@
+// Expert sort of the CVMM path: stable counting sort of expert ids with wavefront ballots.
+//   pass 1  per-wave histograms of 1024-element units (LDS atomics)
+//   pass 2  one workgroup: per-expert totals -> offsets[E+1]; per-unit bases in place
+//   pass 3  per wave: rank every element among equal keys of its 64-lane batch with a
+//           match-any built from ballots over the key bits, add the running per-key base kept
+//           in LDS, scatter (sorted id, flat index, flat index / k)
+// Stable by construction: batches, units and lanes are all visited in ascending flat index.
+#pragma once
+#include "common.h"
+
+namespace amoe {
+
+constexpr int kSelUnit = 1024;      // elements per wave
+constexpr int kSelMaxExperts = 2048;
+
+struct SelParams {
+  const void* sel; int sel_is_i64;
+  long long M; int E, k, n_units, key_bits;
+  int32_t* sel_sorted; int32_t* perm; int32_t* in_index; int32_t* offsets; int32_t* bad_flag;
+  int32_t* unit_hist;               // workspace [n_units][E]
+};
+
+__device__ __forceinline__ int sel_key(const SelParams& p, long long i, bool& bad) {
+  long long v = p.sel_is_i64 ? static_cast<const long long*>(p.sel)[i]
+                             : (long long)static_cast<const int32_t*>(p.sel)[i];
+  bad = v < 0 || v >= p.E;
+  if (v < 0) v = 0;                      // out-of-range ids are flagged and clamped
+  if (v >= p.E) v = p.E - 1;
+  return (int)v;
+}
+
+__global__ __launch_bounds__(kThreads) void sel_hist_kernel(const SelParams p) {
+  __shared__ int hist[4 * kSelMaxExperts];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 4 * p.E; i += kThreads) hist[i] = 0;
+  __syncthreads();
+  const int unit = blockIdx.x * 4 + wave;
+  bool any_bad = false;
+  if (unit < p.n_units) {
+    for (int it = 0; it < kSelUnit / 64; it++) {
+      const long long i = (long long)unit * kSelUnit + it * 64 + lane;
+      if (i < p.M) {
+        bool bad;
+        const int key = sel_key(p, i, bad);
+        any_bad |= bad;
+        atomicAdd(&hist[wave * p.E + key], 1);
+      }
+    }
+  }
+  if (any_bad && p.bad_flag != nullptr) atomicOr(p.bad_flag, 1);
+  __syncthreads();
+  for (int w = 0; w < 4; w++) {
+    const int u = blockIdx.x * 4 + w;
+    if (u < p.n_units)
+      for (int e = tid; e < p.E; e += kThreads) p.unit_hist[(long long)u * p.E + e] = hist[w * p.E + e];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void sel_scan_kernel(const SelParams p) {
+  __shared__ int wave_sums[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per = (p.E + kThreads - 1) / kThreads;
+  const int e0 = tid * per;
+  int mine = 0;
+  for (int j = 0; j < per; j++) {
+    const int e = e0 + j;
+    if (e < p.E)
+      for (int u = 0; u < p.n_units; u++) mine += p.unit_hist[(long long)u * p.E + e];
+  }
+  int incl = mine;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = wave_shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == 63) wave_sums[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; w++) base += wave_sums[w];
+  int run = base + incl - mine;
+  for (int j = 0; j < per; j++) {
+    const int e = e0 + j;
+    if (e < p.E) {
+      p.offsets[e] = run;
+      for (int u = 0; u < p.n_units; u++) {
+        const int c = p.unit_hist[(long long)u * p.E + e];
+        p.unit_hist[(long long)u * p.E + e] = run;
+        run += c;
+      }
+    }
+  }
+  if (tid == 0) p.offsets[p.E] = (int)p.M;
+}
+
+__global__ __launch_bounds__(kThreads) void sel_scatter_kernel(const SelParams p) {
+  __shared__ int base[4 * kSelMaxExperts];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int w = 0; w < 4; w++) {
+    const int u = blockIdx.x * 4 + w;
+    if (u < p.n_units)
+      for (int e = tid; e < p.E; e += kThreads) base[w * p.E + e] = p.unit_hist[(long long)u * p.E + e];
+  }
+  __syncthreads();
+  const int unit = blockIdx.x * 4 + wave;
+  int* my_base = &base[wave * p.E];
+  const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
+  for (int it = 0; it < kSelUnit / 64; it++) {
+    const long long i = (long long)unit * kSelUnit + it * 64 + lane;
+    const bool valid = unit < p.n_units && i < p.M;
+    bool bad;
+    const int key = valid ? sel_key(p, i, bad) : 0;
+    uint64_t same = wave_ballot(valid);
+    for (int b = 0; b < p.key_bits; b++) {
+      const bool bit = (key >> b) & 1;
+      const uint64_t bal = wave_ballot(valid && bit);
+      same &= bit ? bal : ~bal;
+    }
+    const int rank = popc64(same & lt_mask);
+    const int count = popc64(same);
+    int pos = 0;
+    if (valid) pos = my_base[key] + rank;
+    wave_sync();
+    if (valid && rank == 0) my_base[key] += count;
+    wave_sync();
+    if (valid) {
+      p.sel_sorted[pos] = key;
+      p.perm[pos] = (int)i;
+      p.in_index[pos] = (int)(i / p.k);
+    }
+  }
+}
+
+// offsets[E+1] from sorted ids: position i owns every expert in (sel[i-1], sel[i]].
+__global__ __launch_bounds__(kThreads) void offsets_from_sorted_kernel(const int32_t* __restrict__ sel,
+                                                                        long long M, int E,
+                                                                        int32_t* __restrict__ offsets) {
+  const long long i = (long long)blockIdx.x * kThreads + threadIdx.x;
+  if (i > M) return;
+  const int prev = (i == 0) ? -1 : sel[i - 1];
+  int cur = (i == M) ? E : sel[i];
+  if (cur > E) cur = E;
+  for (int e = prev + 1; e <= cur; e++)
+    if (e >= 0) offsets[e] = (int)i;
+}
+
+}  // namespace amoe

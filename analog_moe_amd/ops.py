@@ -1,0 +1,212 @@
+"""Tensor-level entry points of the CVMM path: allocate outputs with torch, run the HIP
+kernels of libamoe.so on the current stream.
+
+There is no CPU path and no fallback: the library must have been built
+(``python -c "import __graft_entry__ as g; g.build()"``) and every tensor must live on the GPU.
+"""
+from __future__ import annotations
+
+import os
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _abi, raw
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libamoe.so")
+_LIB = None
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def get_lib():
+    """The loaded C-ABI library.  Raises if it has not been built."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build the HIP library first (__graft_entry__.build()); "
+                "analog_moe_amd has no CPU fallback")
+        _LIB = _abi.bind(_LIB_PATH)
+    return _LIB
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("analog_moe_amd runs on the GPU only: got a CPU tensor (there is no CPU path)")
+
+
+def _rows2d(t: torch.Tensor) -> torch.Tensor:
+    t = t.reshape(-1, t.shape[-1])
+    return t if t.stride(1) == 1 else t.contiguous()
+
+
+def _f32c(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    return t.detach().to(torch.float32).contiguous()
+
+
+def _i32c(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    return t.detach().reshape(-1).to(torch.int32).contiguous()
+
+
+# ------------------------------------------------------------------------------ selection
+def prepare_sel(sel: torch.Tensor, n_experts: int, k: int) -> Tuple[torch.Tensor, ...]:
+    """Stable expert sort.  Returns (sel_sorted, perm, in_index = perm // k, offsets[E+1]), int32."""
+    _need_gpu(sel)
+    lib = get_lib()
+    flat = sel.detach().reshape(-1)
+    if flat.dtype not in (torch.int32, torch.int64):
+        flat = flat.to(torch.int64)
+    flat = flat.contiguous()
+    M = flat.numel()
+    dev = flat.device
+    sel_sorted = torch.empty(M, dtype=torch.int32, device=dev)
+    perm = torch.empty(M, dtype=torch.int32, device=dev)
+    in_index = torch.empty(M, dtype=torch.int32, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    ws = torch.empty(max(lib.amoe_prepare_sel_workspace(M, n_experts), 4), dtype=torch.uint8, device=dev)
+    raw.prepare_sel(lib, _stream(flat), flat, n_experts, k, sel_sorted, perm, in_index, offsets, None, ws)
+    return sel_sorted, perm, in_index, offsets
+
+
+def offsets_from_sorted(sel_sorted: torch.Tensor, n_experts: int) -> torch.Tensor:
+    _need_gpu(sel_sorted)
+    s = _i32c(sel_sorted)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=s.device)
+    raw.offsets_from_sorted(get_lib(), _stream(s), s, n_experts, offsets)
+    return offsets
+
+
+# ------------------------------------------------------------------------------ forward
+def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets: torch.Tensor,
+             in_index: torch.Tensor, out_index: Optional[torch.Tensor], n_out_rows: int, *,
+             ir: Optional[torch.Tensor] = None, abs_max: Optional[torch.Tensor] = None, inp_res: float = -1.0,
+             bounds: Optional[Sequence[int]] = None, noise: Optional[torch.Tensor] = None,
+             noise_std: float = 0.0, noise_seed: int = 0, wmax: Optional[torch.Tensor] = None,
+             out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False) -> torch.Tensor:
+    """out[out_index[i]] = analog(x[in_index[i]]) @ w[sel_sorted[i]] -> [n_out_rows, N]."""
+    _need_gpu(x, w, sel_sorted, offsets, in_index, out_index, ir, abs_max, noise, wmax)
+    x2 = _rows2d(x)
+    if w.stride(2) != 1 and w.stride(1) != 1:
+        w = w.contiguous()
+    out = torch.empty((n_out_rows, w.shape[2]), dtype=x2.dtype, device=x2.device)
+    raw.cvmm_fwd(get_lib(), _stream(x2), x2, w, out, sel_sorted, offsets, in_index, out_index, _f32c(ir),
+                 _f32c(abs_max), inp_res, bounds, _f32c(noise), noise_std, noise_seed, _f32c(wmax), out_bound,
+                 out_res, relu)
+    return out
+
+
+def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,
+               g_index: Optional[torch.Tensor], *, ir: Optional[torch.Tensor] = None,
+               bounds: Optional[Sequence[int]] = None) -> torch.Tensor:
+    _need_gpu(x, g, offsets, in_index, g_index, ir)
+    x2, g2 = _rows2d(x), _rows2d(g)
+    grad_w = torch.empty((n_experts, x2.shape[1], g2.shape[1]), dtype=x2.dtype, device=x2.device)
+    raw.cvmm_bwd_w(get_lib(), _stream(x2), x2, g2, grad_w, offsets, in_index, g_index, _f32c(ir), bounds)
+    return grad_w
+
+
+def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index: torch.Tensor,
+               out_index: torch.Tensor, n_out_rows: int, *, x: Optional[torch.Tensor] = None,
+               xf_index: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+               ir: Optional[torch.Tensor] = None, bounds: Optional[Sequence[int]] = None,
+               gradient_relative: bool = True, gradient_scale: float = 1.0, decay: float = 0.0,
+               input_min_percentage: float = 0.95, relu_mask: bool = False):
+    """Returns (grad_x_full [n_out_rows, K], ir_grad [M, n_tiles] or None)."""
+    _need_gpu(g, w, offsets, g_index, out_index, x, xf_index, gate, ir)
+    lib = get_lib()
+    g2 = _rows2d(g)
+    if w.stride(2) != 1:
+        w = w.contiguous()
+    E, K, N = w.shape
+    M = g_index.numel()
+    n_tiles = 1 if bounds is None else len(bounds) - 1
+    full = torch.empty((n_out_rows, K), dtype=g2.dtype, device=g2.device)
+    x2 = None if x is None else _rows2d(x)
+    ir32 = _f32c(ir)
+    ir_grad = ws = None
+    if ir32 is not None:
+        ir_grad = torch.empty((M, n_tiles), dtype=torch.float32, device=g2.device)
+        ws = torch.empty(max(raw.bwd_x_workspace_bytes(lib, M, K, n_tiles), 4), dtype=torch.uint8, device=g2.device)
+    gate_c = None if gate is None else gate.detach().reshape(-1).to(g2.dtype).contiguous()
+    raw.cvmm_bwd_x(lib, _stream(g2), g2, w, full, offsets, g_index, out_index, x2, xf_index, gate_c, ir32, ir_grad,
+                   bounds, gradient_relative, gradient_scale, decay, input_min_percentage, relu_mask, ws)
+    return full, ir_grad
+
+
+# ------------------------------------------------------------------------------ companions
+def gate_reduce(z: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """y[t] = sum_j gate[t, j] * z[t, j]; z [T*k, D] (or [..., k, D]), gate [..., k]."""
+    _need_gpu(z, gate)
+    k = gate.shape[-1]
+    z2 = _rows2d(z).contiguous()
+    T, D = z2.shape[0] // k, z2.shape[1]
+    gate_c = gate.detach().reshape(-1).to(z2.dtype).contiguous()
+    y = torch.empty((T, D), dtype=z2.dtype, device=z2.device)
+    raw.gate_reduce(get_lib(), _stream(z2), z2, gate_c, y, T, k, D)
+    return y
+
+
+def ksum(full: torch.Tensor, k: int) -> torch.Tensor:
+    _need_gpu(full)
+    f2 = _rows2d(full).contiguous()
+    T, D = f2.shape[0] // k, f2.shape[1]
+    out = torch.empty((T, D), dtype=f2.dtype, device=f2.device)
+    raw.ksum(get_lib(), _stream(f2), f2, out, T, k, D)
+    return out
+
+
+def gate_grad(z: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:
+    _need_gpu(z, dy)
+    z2, d2 = _rows2d(z).contiguous(), _rows2d(dy).contiguous()
+    T, D = d2.shape
+    out = torch.empty((T, k), dtype=z2.dtype, device=z2.device)
+    raw.gate_grad(get_lib(), _stream(z2), z2, d2, out, T, k, D)
+    return out
+
+
+def row_abs_max(x: torch.Tensor) -> torch.Tensor:
+    _need_gpu(x)
+    x2 = _rows2d(x)
+    out = torch.empty(x2.shape[0], dtype=torch.float32, device=x2.device)
+    raw.row_abs_max(get_lib(), _stream(x2), x2, out)
+    return out
+
+
+def weight_abs_max(w: torch.Tensor, per_channel: bool) -> torch.Tensor:
+    """[E, N] (per channel) or [E, 1] (per expert) max |w|, fp32."""
+    _need_gpu(w)
+    wc = w.detach().contiguous()
+    E, K, N = wc.shape
+    cols = N if per_channel else 1
+    out = torch.empty((E, cols), dtype=torch.float32, device=wc.device)
+    raw.weight_abs_max(get_lib(), _stream(wc), wc, cols, out)
+    return out
+
+
+def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int) -> torch.Tensor:
+    """out[e, t] = sum of v[i, t] over expert e's sorted rows."""
+    _need_gpu(v, offsets)
+    v2 = _f32c(v.reshape(v.shape[0], -1))
+    out = torch.empty((n_experts, v2.shape[1]), dtype=torch.float32, device=v2.device)
+    raw.segment_sum(get_lib(), _stream(v2), v2, offsets, n_experts, v2.shape[1], out)
+    return out
+
+
+def expert_std(x: torch.Tensor, in_index: torch.Tensor, offsets: torch.Tensor, n_experts: int) -> torch.Tensor:
+    _need_gpu(x, in_index, offsets)
+    x2 = _rows2d(x)
+    out = torch.empty(n_experts, dtype=torch.float32, device=x2.device)
+    raw.expert_std(get_lib(), _stream(x2), x2, _i32c(in_index), offsets, n_experts, out)
+    return out

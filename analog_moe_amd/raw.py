@@ -1,0 +1,201 @@
+"""Marshalling layer between tensors and the C ABI (include/amoe.h).
+
+Each function fills the argument struct of one entry point from tensors the caller has
+already allocated and calls it on the given library handle and stream.  Nothing here
+allocates, chooses a device or falls back: it only reads ``data_ptr()``, strides and shapes.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _abi
+from ._abi import AMOE_BF16, AMOE_F32, BwdWArgs, BwdXArgs, FwdArgs, check, set_bounds
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return AMOE_F32
+    if t.dtype == torch.bfloat16:
+        return AMOE_BF16
+    raise TypeError(f"unsupported dtype {t.dtype}: the CVMM kernels take float32 or bfloat16")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: Optional[torch.Tensor], name: str):
+    if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+        raise TypeError(f"{name} must be a contiguous int32 tensor")
+    return t
+
+
+def _f32(t: Optional[torch.Tensor], name: str):
+    if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+        raise TypeError(f"{name} must be a contiguous float32 tensor")
+    return t
+
+
+def _rows(t: torch.Tensor, name: str):
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be 2-D with unit column stride")
+    return t
+
+
+def prepare_sel(lib, stream, sel, E: int, k: int, sel_sorted, perm, in_index, offsets, bad_flag, workspace):
+    if sel.dtype not in (torch.int32, torch.int64) or not sel.is_contiguous():
+        raise TypeError("sel must be a contiguous int32 or int64 tensor")
+    M = sel.numel()
+    for t, n in ((sel_sorted, "sel_sorted"), (perm, "perm"), (in_index, "in_index"), (offsets, "offsets")):
+        _i32(t, n)
+    rc = lib.amoe_prepare_sel(_p(sel), int(sel.dtype == torch.int64), M, E, k, _p(sel_sorted), _p(perm),
+                              _p(in_index), _p(offsets), _p(bad_flag), _p(workspace),
+                              workspace.numel() * workspace.element_size(), stream)
+    check(lib, rc, "amoe_prepare_sel")
+
+
+def offsets_from_sorted(lib, stream, sel_sorted, E: int, offsets):
+    _i32(sel_sorted, "sel_sorted"); _i32(offsets, "offsets")
+    check(lib, lib.amoe_offsets_from_sorted(_p(sel_sorted), sel_sorted.numel(), E, _p(offsets), stream),
+          "amoe_offsets_from_sorted")
+
+
+def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=None, ir=None, abs_max=None,
+             inp_res: float = -1.0, bounds: Optional[Sequence[int]] = None, noise=None, noise_std: float = 0.0,
+             noise_seed: int = 0, wmax=None, out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
+             range_flag=None):
+    """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N]."""
+    _rows(x, "x"); _rows(out, "out")
+    a = FwdArgs()
+    a.dtype = dtype_code(x)
+    if w.dtype != x.dtype or out.dtype != x.dtype:
+        raise TypeError("x, w and out must share one dtype")
+    E, K, N = w.shape
+    if x.shape[1] != K or out.shape[1] != N:
+        raise ValueError("x / w / out shapes do not match")
+    M = in_index.numel()
+    a.M, a.N, a.K, a.E = M, N, K, E
+    a.n_in_rows, a.n_out_rows = x.shape[0], out.shape[0]
+    a.x, a.ldx = _p(x), x.stride(0)
+    a.w, a.w_stride_e, a.w_stride_k, a.w_stride_n = _p(w), w.stride(0), w.stride(1), w.stride(2)
+    a.out, a.ldo = _p(out), out.stride(0)
+    a.sel_sorted, a.offsets = _p(_i32(sel_sorted, "sel_sorted")), _p(_i32(offsets, "offsets"))
+    a.in_index, a.out_index = _p(_i32(in_index, "in_index")), _p(_i32(out_index, "out_index"))
+    set_bounds(a, [0, K] if bounds is None else bounds)
+    if ir is not None and ir.numel() != M * a.n_tiles:
+        raise ValueError("ir must hold one value per sorted position and K-tile")
+    a.ir, a.abs_max, a.inp_res = _p(_f32(ir, "ir")), _p(_f32(abs_max, "abs_max")), float(inp_res)
+    if noise is not None:
+        _f32(noise, "noise")
+        if noise.numel() != a.n_tiles * out.shape[0] * N:
+            raise ValueError("noise must be [n_tiles, out rows, N]")
+        a.noise, a.noise_tile_stride, a.ldnoise = _p(noise), out.shape[0] * N, N
+    a.noise_std, a.noise_seed = float(noise_std), int(noise_seed) & 0xFFFFFFFFFFFFFFFF
+    if wmax is not None:
+        _f32(wmax, "wmax")
+        a.wmax, a.wmax_cols = _p(wmax), wmax.numel() // E
+    a.out_bound, a.out_res = float(out_bound), float(out_res)
+    a.relu, a.range_flag = int(bool(relu)), _p(range_flag)
+    check(lib, lib.amoe_cvmm_fwd(C.byref(a), stream), "amoe_cvmm_fwd")
+
+
+def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=None,
+               bounds: Optional[Sequence[int]] = None):
+    """x [*, K]; g [*, N]; grad_w [E, K, N] contiguous."""
+    _rows(x, "x"); _rows(g, "g")
+    if not grad_w.is_contiguous():
+        raise ValueError("grad_w must be contiguous")
+    a = BwdWArgs()
+    a.dtype = dtype_code(x)
+    if g.dtype != x.dtype or grad_w.dtype != x.dtype:
+        raise TypeError("x, g and grad_w must share one dtype")
+    E, K, N = grad_w.shape
+    if x.shape[1] != K or g.shape[1] != N:
+        raise ValueError("x / g / grad_w shapes do not match")
+    a.M, a.N, a.K, a.E = in_index.numel(), N, K, E
+    a.x, a.ldx, a.g, a.ldg, a.grad_w = _p(x), x.stride(0), _p(g), g.stride(0), _p(grad_w)
+    a.offsets, a.in_index, a.g_index = _p(_i32(offsets, "offsets")), _p(_i32(in_index, "in_index")), \
+        _p(_i32(g_index, "g_index"))
+    set_bounds(a, [0, K] if bounds is None else bounds)
+    a.ir = _p(_f32(ir, "ir"))
+    check(lib, lib.amoe_cvmm_bwd_w(C.byref(a), stream), "amoe_cvmm_bwd_w")
+
+
+def bwd_x_workspace_bytes(lib, M: int, K: int, n_tiles: int) -> int:
+    return lib.amoe_bwd_x_workspace(M, K, n_tiles)
+
+
+def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=None, xf_index=None, gate=None,
+               ir=None, ir_grad=None, bounds: Optional[Sequence[int]] = None, gradient_relative: bool = True,
+               gradient_scale: float = 1.0, decay: float = 0.0, input_min_percentage: float = 0.95,
+               relu_mask: bool = False, workspace=None):
+    """g [*, N]; w [E, K, N] with N contiguous; grad_x_full [R_out, K]; x [*, K] forward input."""
+    _rows(g, "g"); _rows(grad_x_full, "grad_x_full")
+    a = BwdXArgs()
+    a.dtype = dtype_code(g)
+    E, K, N = w.shape
+    if w.stride(2) != 1:
+        raise ValueError("w must have its last dimension contiguous")
+    if g.shape[1] != N or grad_x_full.shape[1] != K:
+        raise ValueError("g / w / grad_x_full shapes do not match")
+    a.M, a.N, a.K, a.E = g_index.numel(), N, K, E
+    a.g, a.ldg = _p(g), g.stride(0)
+    a.w, a.w_stride_e, a.w_stride_k = _p(w), w.stride(0), w.stride(1)
+    a.grad_x_full, a.ldo = _p(grad_x_full), grad_x_full.stride(0)
+    if x is not None:
+        _rows(x, "x")
+        a.x, a.ldx = _p(x), x.stride(0)
+    a.offsets, a.g_index = _p(_i32(offsets, "offsets")), _p(_i32(g_index, "g_index"))
+    a.out_index, a.xf_index = _p(_i32(out_index, "out_index")), _p(_i32(xf_index, "xf_index"))
+    if gate is not None and (gate.dtype != g.dtype or not gate.is_contiguous()):
+        raise TypeError("gate must be contiguous and share the dtype of g")
+    a.gate = _p(gate)
+    set_bounds(a, [0, K] if bounds is None else bounds)
+    a.ir, a.ir_grad = _p(_f32(ir, "ir")), _p(_f32(ir_grad, "ir_grad"))
+    a.gradient_relative, a.gradient_scale = int(bool(gradient_relative)), float(gradient_scale)
+    a.decay, a.input_min_percentage = float(decay), float(input_min_percentage)
+    a.relu_mask = int(bool(relu_mask))
+    if workspace is not None:
+        a.workspace, a.workspace_bytes = _p(workspace), workspace.numel() * workspace.element_size()
+    check(lib, lib.amoe_cvmm_bwd_x(C.byref(a), stream), "amoe_cvmm_bwd_x")
+
+
+def gate_reduce(lib, stream, z, gate, y, T: int, k: int, D: int):
+    check(lib, lib.amoe_gate_reduce(dtype_code(z), _p(z), _p(gate), _p(y), T, k, D, stream), "amoe_gate_reduce")
+
+
+def ksum(lib, stream, full, out, T: int, k: int, D: int):
+    check(lib, lib.amoe_ksum(dtype_code(full), _p(full), _p(out), T, k, D, stream), "amoe_ksum")
+
+
+def gate_grad(lib, stream, z, dy, grad_gate, T: int, k: int, D: int):
+    check(lib, lib.amoe_gate_grad(dtype_code(z), _p(z), _p(dy), _p(grad_gate), T, k, D, stream), "amoe_gate_grad")
+
+
+def row_abs_max(lib, stream, x, out):
+    _rows(x, "x")
+    check(lib, lib.amoe_row_abs_max(dtype_code(x), _p(x), x.stride(0), x.shape[0], x.shape[1],
+                                    _p(_f32(out, "abs_max")), stream), "amoe_row_abs_max")
+
+
+def weight_abs_max(lib, stream, w, cols: int, out):
+    if not w.is_contiguous():
+        raise ValueError("w must be contiguous")
+    E, K, N = w.shape
+    check(lib, lib.amoe_weight_abs_max(dtype_code(w), _p(w), E, K, N, cols, _p(_f32(out, "wmax")), stream),
+          "amoe_weight_abs_max")
+
+
+def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out):
+    check(lib, lib.amoe_segment_sum(_p(_f32(v, "v")), _p(_i32(offsets, "offsets")), E, n_tiles,
+                                    _p(_f32(out, "out")), stream), "amoe_segment_sum")
+
+
+def expert_std(lib, stream, x, in_index, offsets, E: int, out):
+    _rows(x, "x")
+    check(lib, lib.amoe_expert_std(dtype_code(x), _p(x), x.stride(0), x.shape[1], _p(_i32(in_index, "in_index")),
+                                   _p(_i32(offsets, "offsets")), E, _p(_f32(out, "out")), stream),
+          "amoe_expert_std")

@@ -1,0 +1,204 @@
+/* amoe.h -- C ABI of the MI355X-native CVMM path of Analog-MoE (libamoe.so).
+ *
+ * Every entry point is asynchronous on the HIP stream it is given, never synchronises the
+ * host, never allocates or frees device memory and keeps no pointer after it returns: the
+ * caller owns every buffer, including the workspace.  Return value: 0 on success, a negative
+ * AMOE_E* code when the arguments are rejected on the host (nothing was launched), or a
+ * positive hipError_t when a launch failed.  All device pointers must be 4-byte aligned;
+ * 16-byte aligned rows make the kernels take their vector paths.
+ *
+ * The functions replace, one for one, the Triton launchers and the eager glue of the
+ * reference's analog_moe/triton_src/cvmm.py (cited per function, file:line).  A nullable
+ * pointer set to NULL switches the feature off; that replaces the reference's
+ * `torch.tensor(-1)` sentinels (cvmm.py:585-598, 676-681).
+ */
+#ifndef AMOE_H
+#define AMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AMOE_VERSION 100
+#define AMOE_MAX_TILES 16   /* K-tiles per projection (max_input_size splitting) */
+
+enum { AMOE_F32 = 0, AMOE_BF16 = 1 };
+
+enum {
+  AMOE_OK = 0,
+  AMOE_EINVAL = -1,       /* a size, stride or scalar is out of range */
+  AMOE_ENULL = -2,        /* a required pointer is NULL */
+  AMOE_ESHAPE = -3,       /* sizes are inconsistent with each other */
+  AMOE_EALIGN = -4,       /* a pointer is not 4-byte aligned */
+  AMOE_EWORKSPACE = -5,   /* workspace too small */
+  AMOE_EUNSUPPORTED = -6  /* valid request this build does not implement */
+};
+
+int amoe_version(void);
+const char* amoe_strerror(int rc);
+
+/* ---------------------------------------------------------------------------------------
+ * Selection: stable sort of expert ids, index and offset build.
+ * Replaces cvmm_prepare_sel (cvmm.py:31-34: `ssel, perm = sel.flatten().sort()`) and the
+ * second argsort of the backward (cvmm.py:850).  Tie order is fixed: ascending flat index.
+ *   sel        [M] expert id of flat (token, head) position, int32 or int64 (sel_is_i64)
+ *   sel_sorted [M] ascending ids;  perm [M] flat index of each sorted position (the
+ *   up-projection's out_index);  in_index [M] = perm / k (its sel_index);
+ *   offsets [E+1] first sorted position of each expert (new: the kernels use it to cut
+ *   row tiles at expert boundaries).  Ids outside [0, E) make the call set *bad_flag != 0
+ *   (device int32, may be NULL) and are sorted as expert E-1. */
+size_t amoe_prepare_sel_workspace(int64_t M, int32_t E);
+int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, int32_t k,
+                     int32_t* sel_sorted, int32_t* perm, int32_t* in_index, int32_t* offsets,
+                     int32_t* bad_flag, void* workspace, size_t workspace_bytes, void* stream);
+
+/* offsets[E+1] from an already sorted id vector, for callers that arrive with the
+ * reference's own CVMMSel (cvmm.py:19-28), which carries no offsets. */
+int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, int32_t* offsets,
+                             void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Forward: out[out_index[i], :] = analog(x[in_index[i], :]) @ w[sel_sorted[i]]  for every
+ * sorted position i.  Replaces the launcher cvmm_triton_quantized (cvmm.py:531-631) and
+ * cvmm_kernel (cvmm.py:53-231).  Per K-tile t (one tile = the reference's behaviour):
+ *   a = clamp(x, +-ir[i,t]) / ir[i,t] / abs_max[row]; a = rint(a / inp_res) * inp_res
+ *   c = a @ w[e][tile rows, :]  (fp32 accumulate);  c += noise;  c = ADC(c)
+ *   c *= abs_max[row];  c *= ir[i,t];  out += c
+ * The K-tile split, the ADC and the in-kernel noise generator are this library's own
+ * extensions (the reference asserts them off: moe_layer_aihwkit_lightning.py:152-160).
+ */
+typedef struct amoe_fwd_args {
+  int32_t dtype;                 /* AMOE_F32 / AMOE_BF16: type of x, w, out */
+  int32_t M, N, K, E;            /* sorted rows, output features, input features, experts */
+  int32_t n_in_rows, n_out_rows; /* rows of x / of out (indices are checked against nothing
+                                    on the device; the caller guarantees the ranges) */
+  const void* x;   int64_t ldx;                       /* [n_in_rows, K], row stride ldx */
+  const void* w;   int64_t w_stride_e, w_stride_k, w_stride_n; /* [E, K, N] view; one of
+                                    w_stride_n / w_stride_k must be 1 (cvmm.py:839 passes a
+                                    transposed view) */
+  void* out;       int64_t ldo;                       /* [n_out_rows, N] */
+  const int32_t* sel_sorted;     /* [M] */
+  const int32_t* offsets;        /* [E+1] */
+  const int32_t* in_index;       /* [M] */
+  const int32_t* out_index;      /* [M] or NULL -> in_index (cvmm.py:196-205) */
+  const float* ir;               /* [M, n_tiles] input range per sorted position, or NULL */
+  const float* abs_max;          /* [n_in_rows] or NULL (cvmm.py:124-128, 156-158) */
+  float inp_res;                 /* quantisation step; <= 0: no quantisation */
+  int32_t n_tiles;               /* >= 1 */
+  int32_t tile_bounds[AMOE_MAX_TILES + 1]; /* tile t covers input features [b[t], b[t+1]) */
+  const float* noise;            /* [n_tiles, n_out_rows, N] fp32, already scaled, or NULL */
+  int64_t noise_tile_stride, ldnoise;
+  float noise_std;               /* used when noise == NULL and > 0: generate in the kernel
+                                    noise_std * wmax[e, n] * N(0,1), N even */
+  uint64_t noise_seed;
+  const float* wmax;             /* [E, wmax_cols] max |w| per expert (cols 1) or channel (N) */
+  int32_t wmax_cols;
+  float out_bound, out_res;      /* ADC: clamp to +-out_bound*wmax, max(res,1/res) states;
+                                    out_bound <= 0: off; out_res <= 0: clamp only */
+  int32_t relu;                  /* fuse max(., 0) into the store */
+  int32_t* range_flag;           /* device int32 or NULL: set to 1 if |a| > 1 is met before
+                                    quantising (cvmm.py:162 asserts this) */
+} amoe_fwd_args;
+
+int amoe_cvmm_fwd(const amoe_fwd_args* args, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Weight gradient: grad_w[e] = sum_{i in expert e} clamp(x[in_index[i]], +-ir[i,t])^T
+ *                                                   g[g_index[i]]          -> [E, K, N]
+ * Replaces cvmm_triton_backward + cvmm_backward_kernel3 (cvmm.py:645-696, 254-397).
+ * One workgroup owns one output tile of one expert: no atomics, no pre-zeroing, fixed
+ * summation order.  Experts without rows get zeros (cvmm.py:671). */
+typedef struct amoe_bwd_w_args {
+  int32_t dtype;
+  int32_t M, N, K, E;
+  const void* x;  int64_t ldx;           /* forward input  [*, K] */
+  const void* g;  int64_t ldg;           /* output gradient [*, N] */
+  void* grad_w;                          /* [E, K, N] contiguous, dtype */
+  const int32_t* offsets;                /* [E+1] */
+  const int32_t* in_index;               /* [M] row of x per sorted position */
+  const int32_t* g_index;                /* [M] row of g per sorted position, NULL -> in_index
+                                            (cvmm.py:346-351) */
+  const float* ir;                       /* [M, n_tiles] or NULL */
+  int32_t n_tiles;
+  int32_t tile_bounds[AMOE_MAX_TILES + 1];
+} amoe_bwd_w_args;
+
+int amoe_cvmm_bwd_w(const amoe_bwd_w_args* args, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Input gradient with the clip mask, the input-range gradient and the gate scaling fused
+ * into the store.  Replaces the second cvmm_triton_quantized call of CVMM.backward and the
+ * eager glue after it (cvmm.py:828-881, 884-888):
+ *   G = g[g_index[i], :] @ w[e]^T                          (cvmm.py:835-846)
+ *   ir_grad[i,t] = sum_n min([x>=ir] G gate, 0) - sum_n max([x<=-ir] G gate, 0)   (:863-865)
+ *   ir_grad *= ir * gradient_scale (if gradient_relative)                         (:868-870)
+ *   ir_grad += decay * ir * [mean(|x|<ir) > input_min_percentage]                 (:872-878)
+ *   grad_x_full[out_index[i], :] = G * [|x|<ir] * gate [* (x>0) if relu_mask]     (:881, 888)
+ * x is the forward input of the same call, read at row xf_index[i].
+ * workspace: amoe_bwd_x_workspace(M, K, n_tiles) bytes. */
+typedef struct amoe_bwd_x_args {
+  int32_t dtype;
+  int32_t M, N, K, E;            /* as in the forward call: w is [E, K, N]; output has K columns */
+  const void* g;   int64_t ldg;  /* [*, N] */
+  const void* w;   int64_t w_stride_e, w_stride_k; /* [E, K, N], N contiguous */
+  void* grad_x_full; int64_t ldo;   /* [n_out_rows, K] */
+  const void* x;   int64_t ldx;  /* forward input [*, K]; may be NULL when ir == NULL and
+                                    relu_mask == 0 */
+  const int32_t* offsets;        /* [E+1] */
+  const int32_t* g_index;        /* [M] row of g */
+  const int32_t* out_index;      /* [M] row of grad_x_full */
+  const int32_t* xf_index;       /* [M] row of x */
+  const void* gate;              /* [n_out_rows] dtype, indexed by output row, or NULL */
+  const float* ir;               /* [M, n_tiles] or NULL */
+  float* ir_grad;                /* [M, n_tiles] out (required when ir != NULL) */
+  int32_t n_tiles;
+  int32_t tile_bounds[AMOE_MAX_TILES + 1];
+  int32_t gradient_relative;  float gradient_scale;
+  float decay;  float input_min_percentage;
+  int32_t relu_mask;
+  void* workspace;  size_t workspace_bytes;
+} amoe_bwd_x_args;
+
+size_t amoe_bwd_x_workspace(int64_t M, int32_t K, int32_t n_tiles);
+int amoe_cvmm_bwd_x(const amoe_bwd_x_args* args, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Small row-wise companions of CVMM.forward / CVMM.backward.
+ */
+/* y[t, :] = sum_j gate[t, j] * z[t*k + j, :]   (cvmm.py:757-759) */
+int amoe_gate_reduce(int32_t dtype, const void* z, const void* gate, void* y,
+                     int64_t T, int32_t k, int32_t D, void* stream);
+/* out[t, :] = sum_j full[t*k + j, :]           (cvmm.py:890-891) */
+int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, int32_t D,
+              void* stream);
+/* grad_gate[t*k + j] = <z[t*k + j, :], dy[t, :]>   (cvmm.py:889) */
+int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate,
+                   int64_t T, int32_t k, int32_t D, void* stream);
+/* abs_max[r] = max_n |x[r, n]|                 (cvmm.py:733, 737) */
+int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, int32_t K,
+                     float* abs_max, void* stream);
+/* wmax[e, c] = max |w[e, :, c]| (cols == N) or max |w[e]| (cols == 1)
+ * (moe_layer_aihwkit_lightning.py:480-487) */
+int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N,
+                        int32_t cols, float* wmax, void* stream);
+/* out[e, t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]
+ * (moe_layer_aihwkit_lightning.py:447-448), fixed order. */
+int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles,
+                     float* out, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Per-expert unbiased standard deviation of the routed rows' elements, for input-range
+ * initialisation from data.  Replaces cvmm_std and its two kernels (cvmm.py:400-526).
+ * Returns the exact estimate sqrt(SS/(n-1)); an expert without rows gives -0.0, as the
+ * reference's sqrt(0/-1) does.  out is fp32 [E]. */
+int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K,
+                    const int32_t* in_index, const int32_t* offsets, int32_t E,
+                    float* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AMOE_H */

@@ -1,0 +1,153 @@
+"""CPU parity tests of the HIP kernels' own source, compiled for the host with the stand-in
+headers of tests/emu (one thread per GPU thread).  They check index arithmetic, masking, tile
+scheduling and the analog pro/epilogues against the oracle without a GPU; the matrix
+instruction and LDS-transpose stand-ins reproduce the operand layouts measured on MI355X.
+The product path is untouched: these tests point analog_moe_amd.ops at the host build by
+monkeypatching."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from analog_moe_amd import _abi, ops
+from oracle import cvmm_oracle as O
+from tests import util
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+EMU_SO = os.path.join(HERE, "emu", "libamoe_emu.so")
+
+
+@pytest.fixture(scope="module")
+def emu_ops():
+    src = [os.path.join(HERE, "..", "analog_moe_amd", "csrc", f) for f in os.listdir(
+        os.path.join(HERE, "..", "analog_moe_amd", "csrc")) if f.endswith((".h", ".hip"))]
+    src += [os.path.join(HERE, "emu", "gfx950_intrin.h"), os.path.join(HERE, "emu", "hip", "hip_runtime.h")]
+    if not os.path.exists(EMU_SO) or any(os.path.getmtime(s) > os.path.getmtime(EMU_SO) for s in src):
+        subprocess.run([os.path.join(HERE, "emu", "build_emu.sh")], check=True, capture_output=True)
+    lib = _abi.bind(EMU_SO)
+    saved = (ops._LIB, ops._stream, ops._need_gpu)
+    ops._LIB, ops._stream, ops._need_gpu = lib, (lambda t: None), (lambda *a: None)
+    yield ops
+    ops._LIB, ops._stream, ops._need_gpu = saved
+
+
+@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (66, 4, 2), (1500, 8, 2), (5000, 130, 4)])
+def test_prepare_sel_bit_exact(emu_ops, M, E, k):
+    M -= M % k
+    sel = torch.from_numpy(np.random.default_rng(M).integers(0, E, size=M))
+    got = emu_ops.prepare_sel(sel, E, k)
+    want = O.prepare_sel(sel.numpy(), E, k)
+    for g, w in zip(got, (want.sel_sorted, want.perm, want.in_index, want.offsets)):
+        assert np.array_equal(g.numpy(), w)
+    assert np.array_equal(emu_ops.offsets_from_sorted(got[0], E).numpy(), want.offsets)
+    got32 = emu_ops.prepare_sel(sel.to(torch.int32), E, k)
+    assert np.array_equal(got32[1].numpy(), want.perm)
+
+
+CASES = {
+    # name: (problem kwargs, layer kwargs, dtype, tol)
+    "f32_plain": (dict(T=48, D=128, E=4, F=64, k=2), dict(), "f32", 1e-5),
+    "f32_ir_quant": (dict(T=48, D=128, E=4, F=64, k=2), dict(ir=True, inp_res=1 / 127, decay=0.01,
+                                                              input_min_percentage=0.5), "f32", 1e-5),
+    "f32_ragged_K": (dict(T=40, D=77, E=3, F=30, k=2), dict(ir=True, inp_res=1 / 127), "f32", 1e-5),
+    "f32_split_adc_noise": (dict(T=40, D=96, E=4, F=40, k=2),
+                            dict(ir=True, inp_res=1 / 127, bounds_up=[0, 32, 64, 96], bounds_down=[0, 20, 40],
+                                 out_bound=12.0, out_res=254.0, noise=0.04), "f32", 1e-5),
+    "bf16_plain": (dict(T=48, D=128, E=4, F=64, k=2), dict(), "bf16", 2e-2),
+    "bf16_ir_quant": (dict(T=48, D=128, E=4, F=64, k=2), dict(ir=True, inp_res=1 / 127), "bf16", 2e-2),
+    "bf16_ragged": (dict(T=40, D=76, E=3, F=36, k=2), dict(ir=True, inp_res=1 / 127), "bf16", 2e-2),
+    "bf16_split_adc_noise": (dict(T=40, D=128, E=4, F=48, k=2),
+                             dict(ir=True, inp_res=1 / 127, bounds_up=[0, 64, 128], out_bound=12.0, out_res=254.0,
+                                  noise=0.04), "bf16", 2e-2),
+    "f32_big_tile": (dict(T=200, D=40, E=2, F=136, k=2), dict(ir=True, inp_res=1 / 127), "f32", 1e-5),
+}
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_layer_parity_emulated(emu_ops, name):
+    pk, lk, dtype, tol = CASES[name]
+    lk = dict(lk)
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    pr = util.make_problem(7, dtype=tdt, **pk)
+    E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
+    ir = None
+    if lk.pop("ir", False):
+        nt = max(len(lk.get("bounds_up", [0, 1])), len(lk.get("bounds_down", [0, 1]))) - 1
+        ir = torch.from_numpy(np.random.default_rng(1).uniform(0.7, 2.5, size=(2, E, nt)).astype(np.float32))
+    nstd = lk.pop("noise", 0.0)
+    okw = dict(lk)
+    if nstd:
+        ntu = len(lk.get("bounds_up", [0, 1])) - 1
+        ntd = len(lk.get("bounds_down", [0, 1])) - 1
+        g = torch.Generator().manual_seed(3)
+        wu = pr["keys"].float().abs().amax((1, 2))[pr["idx"].reshape(-1)].reshape(1, -1, 1)
+        wd = pr["values"].float().abs().amax((1, 2))[pr["idx"].reshape(-1)].reshape(1, -1, 1)
+        lk["noise_up"] = (torch.randn(ntu, T * k, F, generator=g) * nstd * wu).contiguous()
+        lk["noise_down"] = (torch.randn(ntd, T * k, D, generator=g) * nstd * wd).contiguous()
+        okw["noise_up"], okw["noise_down"] = lk["noise_up"].numpy(), lk["noise_down"].numpy()
+    if lk.get("out_bound", -1) > 0:
+        okw["wmax_up"] = pr["keys"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
+        okw["wmax_down"] = pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
+    got = util.layer_ops_fwd_bwd(emu_ops, pr, ir, **lk)
+    want = util.layer_oracle(pr, ir, dtype, **okw)
+    util.compare_layer(got, want, tol)
+
+
+def test_generated_noise_matches_counter_oracle(emu_ops):
+    pr = util.make_problem(9, T=40, D=64, E=4, F=32, k=2)
+    ir = torch.full((2, 4, 1), 2.0)
+    kw = dict(inp_res=1 / 127, noise_std=0.04, noise_seed=0x1234567890, backward=False)
+    got = util.layer_ops_fwd_bwd(emu_ops, pr, ir, **kw)
+    kw.pop("backward")
+    want = util.layer_oracle(pr, ir, "f32", backward=False,
+                             wmax_up=pr["keys"].abs().amax((1, 2)).reshape(4, 1).numpy(),
+                             wmax_down=pr["values"].abs().amax((1, 2)).reshape(4, 1).numpy(), **kw)
+    assert util.rel_err(got["scores"].numpy(), want.scores) < 1e-4
+    assert util.rel_err(got["y"].numpy(), want.y) < 1e-4
+    clean = util.layer_ops_fwd_bwd(emu_ops, pr, ir, inp_res=1 / 127, backward=False)
+    assert (got["z"] - clean["z"]).abs().max() > 1e-3
+
+
+def test_companions(emu_ops):
+    pr = util.make_problem(11, T=30, D=70, E=5, F=20, k=2)
+    x = pr["x"]
+    assert torch.equal(emu_ops.row_abs_max(x), x.abs().amax(-1))
+    assert torch.equal(emu_ops.weight_abs_max(pr["keys"], False), pr["keys"].abs().amax((1, 2)).reshape(5, 1))
+    assert torch.equal(emu_ops.weight_abs_max(pr["keys"], True), pr["keys"].abs().amax(1))
+    s = emu_ops.prepare_sel(pr["idx"].clamp(max=3), 5, 2)
+    std = emu_ops.expert_std(x, s[2], s[3], 5)
+    want = O.expert_std(x.numpy(), s[2].numpy(), s[0].numpy(), 5)
+    np.testing.assert_allclose(std.numpy()[:4], want[:4], rtol=1e-5)
+    assert not (std[4] > 0)
+
+
+def test_transposed_weight_view(emu_ops):
+    """cvmm.py:839 hands the forward launcher `keys.transpose(1, 2)`: k-contiguous weights."""
+    pr = util.make_problem(13, T=30, D=72, E=3, F=40, k=2)
+    s_sorted, perm, in_index, offsets = emu_ops.prepare_sel(pr["idx"], 3, 2)
+    wt = pr["keys"].transpose(1, 2).contiguous().transpose(1, 2)      # [E, D, F] view with D contiguous
+    a = emu_ops.cvmm_fwd(pr["x"], wt, s_sorted, offsets, in_index, perm, 60)
+    b = emu_ops.cvmm_fwd(pr["x"], pr["keys"], s_sorted, offsets, in_index, perm, 60)
+    np.testing.assert_allclose(a.numpy(), b.numpy(), rtol=1e-5, atol=1e-6)
+    wt16 = wt.bfloat16().transpose(1, 2).contiguous().transpose(1, 2)
+    a16 = emu_ops.cvmm_fwd(pr["x"].bfloat16(), wt16, s_sorted, offsets, in_index, perm, 60)
+    b16 = emu_ops.cvmm_fwd(pr["x"].bfloat16(), pr["keys"].bfloat16(), s_sorted, offsets, in_index, perm, 60)
+    assert torch.equal(a16, b16)
+
+
+def test_argument_errors(emu_ops):
+    lib = ops.get_lib()
+    assert lib.amoe_version() == 100
+    assert lib.amoe_cvmm_fwd(None, None) == -2
+    a = _abi.FwdArgs()
+    a.dtype = 7
+    assert lib.amoe_cvmm_fwd(a, None) == -1
+    pr = util.make_problem(1, T=8, D=16, E=2, F=8, k=2)
+    s_sorted, perm, in_index, offsets = emu_ops.prepare_sel(pr["idx"], 2, 2)
+    with pytest.raises(_abi.AmoeError, match="inconsistent sizes"):
+        emu_ops.cvmm_fwd(pr["x"], pr["keys"], s_sorted, offsets, in_index, perm, 16, bounds=[0, 8, 15])
+    with pytest.raises(_abi.AmoeError):
+        emu_ops.cvmm_fwd(pr["x"], pr["keys"], s_sorted, offsets, in_index, perm, 16, out_bound=12.0)  # no wmax
+    assert b"workspace" in lib.amoe_strerror(-5)

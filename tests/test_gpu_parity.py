@@ -1,0 +1,137 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (analog_moe_amd.ops ->
+libamoe.so), against the CPU oracle on the same seeded inputs.
+Tolerances: selection bit-exact; fp32 1e-5 and bf16 2e-2 relative to the scale of the
+reference tensor (max |a-b| / max |b|)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cvmm_oracle as O
+from tests import util
+from tests.test_emu_kernels import CASES
+
+pytestmark = pytest.mark.gpu
+TOL = {"f32": 1e-5, "bf16": 2e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from analog_moe_amd import ops as _ops
+    _ops.get_lib()          # fails loudly when libamoe.so has not been built
+    return _ops
+
+
+def _to(pr, dev="cuda"):
+    return {n: t.to(dev) for n, t in pr.items()}
+
+
+@pytest.mark.parametrize("M,E,k,skew", [(0, 4, 1, False), (1, 1, 1, False), (512, 8, 2, False), (32768, 16, 4, False),
+                                        (131072, 64, 8, False), (131072, 128, 4, True), (100003, 1000, 1, True),
+                                        (3 * 4099, 2048, 3, False)])
+def test_prepare_sel_bit_exact(ops, M, E, k, skew):
+    rng = np.random.default_rng(M + E)
+    if skew:
+        p = np.arange(1, E + 1) ** -1.2
+        sel = rng.choice(E, size=M, p=p / p.sum())
+    else:
+        sel = rng.integers(0, E, size=M)
+    print(f"prepare_sel M={M} E={E} k={k} skew={skew}", flush=True)
+    got = ops.prepare_sel(torch.from_numpy(sel).cuda(), E, k)
+    want = O.prepare_sel(sel, E, k)
+    for g, w in zip(got, (want.sel_sorted, want.perm, want.in_index, want.offsets)):
+        assert np.array_equal(g.cpu().numpy(), w)
+    assert np.array_equal(ops.offsets_from_sorted(got[0], E).cpu().numpy(), want.offsets)
+    got32 = ops.prepare_sel(torch.from_numpy(sel.astype(np.int32)).cuda(), E, k)
+    assert np.array_equal(got32[1].cpu().numpy(), want.perm)
+
+
+def _run_case(ops, pk, lk, dtype, seed=7, routing="router"):
+    lk = dict(lk)
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    pr = util.make_problem(seed, dtype=tdt, routing=routing, **pk)
+    E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
+    ir = None
+    irspec = lk.pop("ir", False)
+    if irspec:
+        nt = max(len(lk.get("bounds_up", [0, 1])), len(lk.get("bounds_down", [0, 1]))) - 1
+        if irspec is True:
+            ir = torch.from_numpy(np.random.default_rng(1).uniform(0.7, 2.5, size=(2, E, nt)).astype(np.float32))
+        else:
+            ir = torch.full((2, E, nt), float(irspec))
+    nstd = lk.pop("noise", 0.0)
+    okw = dict(lk)
+    if nstd:
+        ntu = len(lk.get("bounds_up", [0, 1])) - 1
+        ntd = len(lk.get("bounds_down", [0, 1])) - 1
+        g = torch.Generator().manual_seed(3)
+        wu = pr["keys"].float().abs().amax((1, 2))[pr["idx"].reshape(-1)].reshape(1, -1, 1)
+        wd = pr["values"].float().abs().amax((1, 2))[pr["idx"].reshape(-1)].reshape(1, -1, 1)
+        nu = (torch.randn(ntu, T * k, F, generator=g) * nstd * wu).contiguous()
+        nd = (torch.randn(ntd, T * k, D, generator=g) * nstd * wd).contiguous()
+        lk["noise_up"], lk["noise_down"] = nu.cuda(), nd.cuda()
+        okw["noise_up"], okw["noise_down"] = nu.numpy(), nd.numpy()
+    if lk.get("out_bound", -1) > 0:
+        okw["wmax_up"] = pr["keys"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
+        okw["wmax_down"] = pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
+    got = util.layer_ops_fwd_bwd(ops, _to(pr), None if ir is None else ir.cuda(), **lk)
+    torch.cuda.synchronize()
+    want = util.layer_oracle(pr, ir, dtype, **okw)
+    return util.compare_layer(got, want, TOL[dtype])
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_layer_parity_small(ops, name):
+    pk, lk, dtype, _ = CASES[name]
+    print("case", name, flush=True)
+    print(_run_case(ops, pk, lk, dtype))
+
+
+def test_config1_cpu_runnable_layer(ops):
+    """BASELINE config 1: D=128, E=8, F=64, k=2, 4x64 tokens, fp32, fixed input range 3.0,
+    8-bit input quantisation, no noise, 8-bit ADC; forward + backward."""
+    print("config 1", flush=True)
+    errs = _run_case(ops, dict(T=256, D=128, E=8, F=64, k=2),
+                     dict(ir=3.0, inp_res=1 / 127, out_bound=12.0, out_res=254.0), "f32", seed=0)
+    print(errs)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_config2_paper_scale_layer(ops, dtype):
+    """BASELINE config 2: D=412 (not a multiple of the vector width), E=16, F=128, k=4,
+    32x256 tokens, per-expert input ranges, 8-bit DAC/ADC, injected output noise 0.04 * max|W|."""
+    print("config 2", dtype, flush=True)
+    errs = _run_case(ops, dict(T=8192, D=412, E=16, F=128, k=4),
+                     dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01,
+                          input_min_percentage=0.9), dtype, seed=0)
+    print(errs)
+
+
+def test_generated_noise_matches_counter_oracle(ops):
+    pr = util.make_problem(9, T=500, D=256, E=8, F=128, k=2)
+    ir = torch.full((2, 8, 1), 2.0)
+    kw = dict(inp_res=1 / 127, noise_std=0.04, noise_seed=0x1234567890)
+    got = util.layer_ops_fwd_bwd(ops, _to(pr), ir.cuda(), backward=False, **kw)
+    want = util.layer_oracle(pr, ir, "f32", backward=False,
+                             wmax_up=pr["keys"].abs().amax((1, 2)).reshape(8, 1).numpy(),
+                             wmax_down=pr["values"].abs().amax((1, 2)).reshape(8, 1).numpy(), **kw)
+    # hardware log / sin / cos differ from libm in the last bits
+    assert util.rel_err(got["scores"].cpu().numpy(), want.scores) < 1e-4
+    assert util.rel_err(got["y"].cpu().numpy(), want.y) < 1e-4
+
+
+def test_companions(ops):
+    pr = _to(util.make_problem(11, T=300, D=70, E=5, F=20, k=2))
+    x = pr["x"]
+    assert torch.equal(ops.row_abs_max(x), x.abs().amax(-1))
+    assert torch.equal(ops.weight_abs_max(pr["keys"], False), pr["keys"].abs().amax((1, 2)).reshape(5, 1))
+    assert torch.equal(ops.weight_abs_max(pr["keys"], True), pr["keys"].abs().amax(1))
+    s = ops.prepare_sel(pr["idx"].clamp(max=3), 5, 2)
+    std = ops.expert_std(x, s[2], s[3], 5).cpu().numpy()
+    want = O.expert_std(x.cpu().numpy(), s[2].cpu().numpy(), s[0].cpu().numpy(), 5)
+    np.testing.assert_allclose(std[:4], want[:4], rtol=1e-5)
+    assert not (std[4] > 0)
+
+
+def test_cpu_tensors_are_rejected(ops):
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.prepare_sel(torch.zeros(4, dtype=torch.int64), 2, 1)

@@ -1,0 +1,123 @@
+"""Shared by the CPU (emulated) and GPU parity tests: builds seeded problems, runs the layer
+through analog_moe_amd.ops and through the oracle, and compares."""
+import numpy as np
+import torch
+
+from oracle import cvmm_oracle as O
+
+
+def make_problem(seed, T, D, E, F, k, dtype=torch.float32, routing="router", device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, D, generator=g)
+    keys = torch.randn(E, D, F, generator=g) / D ** 0.5
+    values = torch.randn(E, F, D, generator=g) / F ** 0.5
+    if routing == "router":
+        router = torch.randn(E, D, generator=g) / D ** 0.5
+        gate, idx = torch.sigmoid(x @ router.t()).topk(k, dim=-1, sorted=False)
+    elif routing == "uniform":      # every expert gets exactly T*k/E rows
+        base = (torch.arange(T * k) % E).reshape(T, k)
+        shift = torch.randint(0, E, (T, 1), generator=g)
+        idx = (base + shift) % E
+        gate = torch.rand(T, k, generator=g) * 0.5 + 0.25
+    elif routing == "zipf":         # logits biased so that load follows Zipf(1.2)
+        p = torch.arange(1, E + 1, dtype=torch.float32) ** -1.2
+        logits = torch.randn(T, E, generator=g) + torch.log(p / p.sum())
+        gate, idx = torch.sigmoid(logits).topk(k, dim=-1, sorted=False)
+    else:
+        raise ValueError(routing)
+    dy = torch.randn(T, D, generator=g)
+    cast = lambda t: t.to(dtype).to(device)
+    return dict(x=cast(x), keys=cast(keys), values=cast(values), idx=idx.to(device), gate=cast(gate), dy=cast(dy))
+
+
+def np32(t):
+    return None if t is None else t.detach().float().cpu().numpy()
+
+
+def layer_ops_fwd_bwd(ops, pr, ir=None, *, inp_res=-1.0, noise_up=None, noise_down=None, noise_std=0.0,
+                      noise_seed=None, out_bound=-1.0, out_res=-1.0, bounds_up=None, bounds_down=None, decay=0.0,
+                      input_min_percentage=0.95, gradient_relative=True, gradient_scale=1.0, per_channel=False,
+                      backward=True):
+    """The layer of oracle.layer_fwd_bwd, through the kernels.  ir [2, E, n_tiles] tensor or None."""
+    x, keys, values, idx, gate, dy = (pr[n] for n in ("x", "keys", "values", "idx", "gate", "dy"))
+    T, D = x.shape
+    E, _, F = keys.shape
+    k = idx.shape[1]
+    M = T * k
+    sel_sorted, perm, in_index, offsets = ops.prepare_sel(idx, E, k)
+    sel_l = sel_sorted.long()
+    ntu = 1 if bounds_up is None else len(bounds_up) - 1
+    ntd = 1 if bounds_down is None else len(bounds_down) - 1
+    ir_up = ir_dn = None
+    if ir is not None:
+        ir_up = ir[0][sel_l][:, :ntu].contiguous()
+        ir_dn = ir[1][sel_l][:, :ntd].contiguous()
+    need_wmax = out_bound > 0 or (noise_seed is not None and noise_std > 0)
+    wu = ops.weight_abs_max(keys, per_channel) if need_wmax else None
+    wd = ops.weight_abs_max(values, per_channel) if need_wmax else None
+    gen = noise_seed is not None and noise_std > 0
+    p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, inp_res=inp_res, bounds=bounds_up,
+                      noise=noise_up, noise_std=noise_std if gen else 0.0, noise_seed=noise_seed or 0, wmax=wu,
+                      out_bound=out_bound, out_res=out_res, relu=True)
+    z = ops.cvmm_fwd(p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn, inp_res=inp_res, bounds=bounds_down,
+                     noise=noise_down, noise_std=noise_std if gen else 0.0, noise_seed=(noise_seed or 0) + 1,
+                     wmax=wd, out_bound=out_bound, out_res=out_res)
+    y = ops.gate_reduce(z, gate)
+    res = dict(y=y, scores=p1, z=z, sel_sorted=sel_sorted, perm=perm, in_index=in_index, offsets=offsets)
+    if not backward:
+        return res
+    irkw = dict(gradient_relative=gradient_relative, gradient_scale=gradient_scale, decay=decay,
+                input_min_percentage=input_min_percentage)
+    # down-projection backward (cvmm.py:785-889)
+    g_w = (gate.reshape(-1, 1) * dy.repeat_interleave(k, dim=0)).to(dy.dtype)
+    res["grad_values"] = ops.cvmm_bwd_w(p1, g_w, E, offsets, perm, None, ir=ir_dn, bounds=bounds_down)
+    g_tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+    gp1, irg_dn = ops.cvmm_bwd_x(dy, values, offsets, g_tok, perm, M, x=p1, xf_index=perm, gate=gate, ir=ir_dn,
+                                 bounds=bounds_down, relu_mask=True, **irkw)
+    res["grad_gate"] = ops.gate_grad(z, dy, k)
+    # up-projection backward
+    res["grad_keys"] = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=bounds_up)
+    full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
+                                  bounds=bounds_up, **irkw)
+    res["grad_x"] = ops.ksum(full, k)
+    res["grad_p1"] = gp1
+    if ir is not None:
+        nt = ir.shape[2]
+        gi = torch.zeros(2, E, nt, device=x.device)
+        gi[0, :, :ntu] = ops.segment_sum(irg_up, offsets, E)
+        gi[1, :, :ntd] = ops.segment_sum(irg_dn, offsets, E)
+        res["grad_ir"] = gi
+        res["ir_grad_up"], res["ir_grad_dn"] = irg_up, irg_dn
+    return res
+
+
+def layer_oracle(pr, ir=None, dtype="f32", backward=True, **kw):
+    return O.layer_fwd_bwd(np32(pr["x"]), np32(pr["keys"]), np32(pr["values"]), pr["idx"].cpu().numpy(),
+                           np32(pr["gate"]), None if ir is None else np32(ir), np32(pr["dy"]) if backward else None,
+                           dtype=dtype, **kw)
+
+
+def rel_err(a, b):
+    """max |a-b| / max |b|: error relative to the scale of the reference tensor."""
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def compare_layer(got, want, tol, check_sel=True, skip=()):
+    """got: dict from layer_ops_fwd_bwd; want: LayerOracle."""
+    if check_sel:
+        assert np.array_equal(got["sel_sorted"].cpu().numpy(), want.sel.sel_sorted)
+        assert np.array_equal(got["perm"].cpu().numpy(), want.sel.perm)
+        assert np.array_equal(got["in_index"].cpu().numpy(), want.sel.in_index)
+        assert np.array_equal(got["offsets"].cpu().numpy(), want.sel.offsets)
+    pairs = [("scores", want.scores), ("z", want.z), ("y", want.y), ("grad_values", want.grad_values),
+             ("grad_keys", want.grad_keys), ("grad_x", want.grad_x), ("grad_gate", want.grad_gate),
+             ("grad_ir", want.grad_ir)]
+    errs = {}
+    for name, ref in pairs:
+        if ref is None or name not in got or name in skip:
+            continue
+        errs[name] = rel_err(np32(got[name]).reshape(ref.shape), ref)
+    bad = {n: e for n, e in errs.items() if not e <= tol}
+    assert not bad, f"relative error above {tol}: {bad} (all: {errs})"
+    return errs
