@@ -469,10 +469,17 @@ def layer_fwd_bwd(x, keys, values, sel_idx, sel_val, ir=None, dy=None, *, inp_re
                   noise_up=None, noise_down=None, wmax_up=None, wmax_down=None,
                   noise_std=0.0, noise_seed=None, out_bound=-1.0, out_res=-1.0,
                   bounds_up=None, bounds_down=None, decay=0.0, input_min_percentage=0.95,
-                  gradient_relative=True, gradient_scale=1.0, dtype="f32") -> LayerOracle:
+                  gradient_relative=True, gradient_scale=1.0, dtype="f32",
+                  scores_override=None, z_override=None) -> LayerOracle:
     """SigmaMoE FFN with analog experts: y[t] = sum_h gate[t,h] * A(relu(A(x[t], keys[e])), values[e])
     (per-token form in test_moe_layer_aihwkit_lightning.py:82-107), built from the CVMM
-    calls of moe_layer_aihwkit_lightning.py:384-410, 494-506.  ir: [2, E, n_tiles] or None."""
+    calls of moe_layer_aihwkit_lightning.py:384-410, 494-506.  ir: [2, E, n_tiles] or None.
+
+    ``scores_override`` / ``z_override``: continue from these stage outputs instead of the
+    oracle's own (the returned ``scores`` / ``z`` stay the oracle's).  An output quantiser
+    turns a last-bit difference in the accumulation into a whole ADC step for the few values
+    that sit on a rounding boundary; checking stage by stage keeps such flips from leaking
+    into the comparison of the later stages."""
     x = np.asarray(x, dtype=F32)
     T, D = x.shape
     E, _, Fdim = keys.shape
@@ -490,12 +497,18 @@ def layer_fwd_bwd(x, keys, values, sel_idx, sel_val, ir=None, dy=None, *, inp_re
     p1 = cvmm_fwd(x, s.in_index, s.sel_sorted, keys, inp_res, ir_up, s.perm, None, noise_up,
                   bounds=bu, wmax=wmax_up, out_bound=out_bound, out_res=out_res,
                   noise_std=noise_std, noise_seed=seed_up, dtype=dtype, relu=True)
+    p1_own = p1
+    if scores_override is not None:
+        p1 = np.asarray(scores_override, dtype=F32).reshape(p1.shape)
     z = cvmm_fwd(p1, s.perm, s.sel_sorted, values, inp_res, ir_dn, None, None, noise_down,
                  bounds=bd, wmax=wmax_down, out_bound=out_bound, out_res=out_res,
                  noise_std=noise_std, noise_seed=seed_dn, dtype=dtype)
+    z_own = z
+    if z_override is not None:
+        z = np.asarray(z_override, dtype=F32).reshape(z.shape)
     gate = _cast(np.asarray(sel_val, dtype=F32), dtype)
     y = gate_reduce(z, gate, dtype)
-    res = LayerOracle(y, p1, z, s)
+    res = LayerOracle(y, p1_own, z_own, s)
     if dy is None:
         return res
     kw = dict(k=k, decay=decay, input_min_percentage=input_min_percentage,

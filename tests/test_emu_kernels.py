@@ -91,8 +91,8 @@ def test_layer_parity_emulated(emu_ops, name):
         okw["wmax_up"] = pr["keys"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
         okw["wmax_down"] = pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
     got = util.layer_ops_fwd_bwd(emu_ops, pr, ir, **lk)
-    want = util.layer_oracle(pr, ir, dtype, **okw)
-    util.compare_layer(got, want, tol)
+    want = util.layer_oracle(pr, ir, dtype, got=got, **okw)
+    util.compare_layer(got, want, tol, adc_step=util.adc_steps(pr, ir, lk))
 
 
 def test_generated_noise_matches_counter_oracle(emu_ops):

@@ -75,8 +75,8 @@ def _run_case(ops, pk, lk, dtype, seed=7, routing="router"):
         okw["wmax_down"] = pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy()
     got = util.layer_ops_fwd_bwd(ops, _to(pr), None if ir is None else ir.cuda(), **lk)
     torch.cuda.synchronize()
-    want = util.layer_oracle(pr, ir, dtype, **okw)
-    return util.compare_layer(got, want, TOL[dtype])
+    want = util.layer_oracle(pr, ir, dtype, got=got, **okw)
+    return util.compare_layer(got, want, TOL[dtype], adc_step=util.adc_steps(pr, ir, lk))
 
 
 @pytest.mark.parametrize("name", list(CASES))
