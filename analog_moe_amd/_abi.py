@@ -20,7 +20,7 @@ class FwdArgs(C.Structure):
         ("w", P), ("w_stride_e", C.c_int64), ("w_stride_k", C.c_int64), ("w_stride_n", C.c_int64),
         ("out", P), ("ldo", C.c_int64),
         ("sel_sorted", P), ("offsets", P), ("in_index", P), ("out_index", P),
-        ("ir", P), ("abs_max", P), ("inp_res", C.c_float),
+        ("ir", P), ("ir_by_expert", C.c_int32), ("abs_max", P), ("inp_res", C.c_float),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
         ("noise", P), ("noise_tile_stride", C.c_int64), ("ldnoise", C.c_int64),
         ("noise_std", C.c_float), ("noise_seed", C.c_uint64),
@@ -34,7 +34,8 @@ class BwdWArgs(C.Structure):
     _fields_ = [
         ("dtype", C.c_int32), ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("E", C.c_int32),
         ("x", P), ("ldx", C.c_int64), ("g", P), ("ldg", C.c_int64), ("grad_w", P),
-        ("offsets", P), ("in_index", P), ("g_index", P), ("ir", P),
+        ("offsets", P), ("in_index", P), ("g_index", P), ("ir", P), ("ir_by_expert", C.c_int32),
+        ("g_scale", P),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
     ]
 
@@ -47,7 +48,7 @@ class BwdXArgs(C.Structure):
         ("grad_x_full", P), ("ldo", C.c_int64),
         ("x", P), ("ldx", C.c_int64),
         ("offsets", P), ("g_index", P), ("out_index", P), ("xf_index", P),
-        ("gate", P), ("ir", P), ("ir_grad", P),
+        ("gate", P), ("ir", P), ("ir_by_expert", C.c_int32), ("ir_grad", P),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
         ("gradient_relative", C.c_int32), ("gradient_scale", C.c_float),
         ("decay", C.c_float), ("input_min_percentage", C.c_float),

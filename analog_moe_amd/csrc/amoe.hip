@@ -145,7 +145,8 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   for (int t = 0; t <= a->n_tiles; t++) p.kd_bounds[t] = a->tile_bounds[t];
   p.n_col_tiles = 1; p.col_bounds[0] = 0; p.col_bounds[1] = a->N;
   p.n_col_blocks = count_col_blocks(p.col_bounds, 1);
-  p.ir = a->ir; p.ir_cols = a->n_tiles; p.abs_max = a->abs_max; p.inp_res = a->inp_res;
+  p.ir = a->ir; p.ir_cols = a->n_tiles; p.ir_by_expert = a->ir_by_expert; p.abs_max = a->abs_max;
+  p.inp_res = a->inp_res;
   p.noise = a->noise; p.noise_ts = a->noise_tile_stride; p.ldnoise = a->ldnoise;
   p.noise_std = a->noise_std; p.seed = a->noise_seed;
   p.wmax = a->wmax; p.wmax_cols = a->wmax_cols;
@@ -178,14 +179,14 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   if (a->M > 0 && (a->ldx < a->K || a->ldg < a->N)) return AMOE_ESHAPE;
   const size_t es = esize(a->dtype);
   if (!aligned(a->x, es) || !aligned(a->g, es) || !aligned(a->grad_w, es) || !aligned(a->offsets, 4) ||
-      !aligned(a->in_index, 4) || !aligned(a->g_index, 4) || !aligned(a->ir, 4))
+      !aligned(a->in_index, 4) || !aligned(a->g_index, 4) || !aligned(a->ir, 4) || !aligned(a->g_scale, es))
     return AMOE_EALIGN;
   const int CH = a->dtype == AMOE_F32 ? 4 : 8;
   WgradParams p{};
   p.M = a->M; p.N = a->N; p.K = a->K; p.E = a->E;
   p.x = a->x; p.ldx = a->ldx; p.g = a->g; p.ldg = a->ldg; p.grad_w = a->grad_w;
   p.offsets = a->offsets; p.in_index = a->in_index; p.g_index = a->g_index;
-  p.ir = a->ir; p.n_tiles = a->n_tiles;
+  p.ir = a->ir; p.ir_by_expert = a->ir_by_expert; p.g_scale = a->g_scale; p.n_tiles = a->n_tiles;
   for (int t = 0; t <= a->n_tiles; t++) p.bounds[t] = a->tile_bounds[t];
   p.n_k_blocks = count_col_blocks(p.bounds, p.n_tiles);
   p.n_n_blocks = (a->N + kTileCols - 1) / kTileCols;
@@ -241,7 +242,7 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.n_col_tiles = a->n_tiles;
   for (int t = 0; t <= a->n_tiles; t++) p.col_bounds[t] = a->tile_bounds[t];
   p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles);
-  p.ir = a->ir; p.ir_cols = a->n_tiles; p.inp_res = -1.f;
+  p.ir = a->ir; p.ir_cols = a->n_tiles; p.ir_by_expert = a->ir_by_expert; p.inp_res = -1.f;
   p.xf = a->x; p.ldxf = a->ldx; p.xf_index = a->xf_index; p.gate = a->gate; p.relu_mask = a->relu_mask;
   const int row_tiles = max_row_tiles(a->M, a->E);
   const int grid = row_tiles * p.n_col_blocks;
@@ -264,7 +265,7 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
     f.M = a->M; f.n_tiles = a->n_tiles; f.KD_total = a->K;
     for (int t = 0; t <= a->n_tiles; t++) f.col_bounds[t] = a->tile_bounds[t];
     f.irg_partial = p.irg_partial; f.notclip_count = p.notclip_count; f.n_blocks = grid;
-    f.ir = a->ir; f.ir_grad = a->ir_grad;
+    f.ir = a->ir; f.ir_by_expert = a->ir_by_expert; f.offsets = a->offsets; f.E = a->E; f.ir_grad = a->ir_grad;
     f.relative = a->gradient_relative; f.scale = a->gradient_scale; f.decay = a->decay;
     f.min_pct = a->input_min_percentage;
     hipLaunchKernelGGL(ir_grad_finalize_kernel, dim3((a->M + kThreads - 1) / kThreads), dim3(kThreads), 0, st, f);

@@ -31,7 +31,7 @@ struct RowsParams {
   int n_col_tiles; int col_bounds[kMaxTiles + 1]; // column split (input gradient: K-tiles of x)
   int n_col_blocks;
   // forward
-  const float* ir; int ir_cols; const float* abs_max; float inp_res;
+  const float* ir; int ir_cols; int ir_by_expert; const float* abs_max; float inp_res;
   const float* noise; int64_t noise_ts, ldnoise; float noise_std; uint64_t seed;
   const float* wmax; int wmax_cols; float out_bound, out_half_states; int relu;
   int32_t* range_flag;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int r = row0 + (tid >> 3) + 32 * i;
-      a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)r * p.ir_cols + t] : 1.f;
+      a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
     }
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
         const bool valid = r < row_end;
         const int arow = valid ? p.a_index[r] : 0;
         const int orow = valid ? (p.out_index ? p.out_index[r] : arow) : 0;
-        const float ir_r = (has_ir && valid) ? p.ir[(int64_t)r * p.ir_cols + t] : 1.f;
+        const float ir_r = (has_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
         const float am_r = (has_amax && valid) ? p.abs_max[arow] : 1.f;
 #pragma unroll
         for (int fi = 0; fi < 2; fi++) {
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
       const int orow = valid ? p.out_index[r] : 0;
       const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
       const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
-      const float ir_r = (use_ir && valid) ? p.ir[(int64_t)r * p.ir_cols + colb.tile] : 0.f;
+      const float ir_r = (use_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile] : 0.f;
       float part = 0.f;
 #pragma unroll
       for (int fi = 0; fi < 2; fi++) {
@@ -402,7 +402,7 @@ struct IrFinalizeParams {
   int M, n_tiles, KD_total;      // KD_total = columns of x (for the un-clipped fraction)
   int col_bounds[kMaxTiles + 1];
   const float* irg_partial; const int32_t* notclip_count; int n_blocks;
-  const float* ir; float* ir_grad;
+  const float* ir; int ir_by_expert; const int32_t* offsets; int E; float* ir_grad;
   int relative; float scale, decay, min_pct;
 };
 
@@ -423,13 +423,22 @@ __global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFina
   }
   const int r = blockIdx.x * kThreads + tid;
   if (r >= p.M) return;
+  int ir_row = r;
+  if (p.ir_by_expert) {  // expert of sorted position r: last e with offsets[e] <= r
+    int lo = 0, hi = p.E - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.offsets[mid] <= r) lo = mid; else hi = mid - 1;
+    }
+    ir_row = lo;
+  }
   int cb = 0;
   for (int t = 0; t < p.n_tiles; t++) {
     const int nb = (p.col_bounds[t + 1] - p.col_bounds[t] + kTileCols - 1) / kTileCols;
     float s = 0.f;
     for (int b = 0; b < nb; b++) s += p.irg_partial[(int64_t)(cb + b) * p.M + r];
     cb += nb;
-    const float irv = p.ir[(int64_t)r * p.n_tiles + t];
+    const float irv = p.ir[(int64_t)ir_row * p.n_tiles + t];
     if (p.relative) s = s * irv * p.scale;
     if (p.decay > 0.f) s = s + p.decay * irv * flag;
     p.ir_grad[(int64_t)r * p.n_tiles + t] = s;

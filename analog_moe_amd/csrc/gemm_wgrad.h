@@ -16,7 +16,7 @@ struct WgradParams {
   const void* g; int64_t ldg;
   void* grad_w;
   const int32_t* offsets; const int32_t* in_index; const int32_t* g_index;
-  const float* ir; int n_tiles; int bounds[kMaxTiles + 1];
+  const float* ir; int ir_by_expert; const void* g_scale; int n_tiles; int bounds[kMaxTiles + 1];
   int n_k_blocks, n_n_blocks;
   int x_vec, g_vec, out_vec;
 };
@@ -49,6 +49,7 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
 
   const T* __restrict__ X = static_cast<const T*>(p.x);
   const T* __restrict__ G = static_cast<const T*>(p.g);
+  const T* __restrict__ GS = static_cast<const T*>(p.g_scale);
   const bool has_ir = p.ir != nullptr;
   const int chunk = tid % CPR;
 
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
       nvx = nvx < 0 ? 0 : (nvx > CH ? CH : nvx);
       rx[i] = chunk_load<T>(X + (int64_t)xi * p.ldx + kk, nvx, p.x_vec != 0);
       if (has_ir && ok) {
-        const float rng = p.ir[(int64_t)r * p.n_tiles + kcol.tile];
+        const float rng = p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.n_tiles + kcol.tile];
 #pragma unroll
         for (int j = 0; j < CH; j++) {
           float v = rx[i].v[j];
@@ -86,6 +87,11 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
       int nvg = ok ? n1 - n : 0;
       nvg = nvg < 0 ? 0 : (nvg > CH ? CH : nvg);
       rg[i] = chunk_load<T>(G + (int64_t)gi * p.ldg + n, nvg, p.g_vec != 0);
+      if (GS != nullptr && ok) {
+        const float sc = Elem<T>::load(GS + xi);
+#pragma unroll
+        for (int j = 0; j < CH; j++) rg[i].v[j] *= sc;
+      }
     }
   };
 

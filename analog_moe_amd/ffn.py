@@ -1,0 +1,100 @@
+"""Fused expert feed-forward of the analog SigmaMoE layer as ONE autograd function.
+
+Same arithmetic as two CVMM calls with a ReLU between them (moe_layer_aihwkit_lightning.py:
+384-410, 494-506; cvmm.py:699-897), with the glue folded into the kernels: the ReLU into the
+up-projection's store and the down-projection's input gradient, the gate (x) dy outer product
+into the weight-gradient loader, the per-position input-range gather into a per-expert table,
+and the noise draw into the epilogue.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from . import ops
+
+
+@dataclass
+class FFNConfig:
+    inp_res: float = -1.0                         # kernel step (1/127 for 8 bit); <= 0 off
+    bounds_up: Optional[Sequence[int]] = None     # K-tile bounds of the up-projection
+    bounds_down: Optional[Sequence[int]] = None
+    out_bound: float = -1.0
+    out_res: float = -1.0
+    noise_std: float = 0.0                        # in-kernel noise, in units of max|W|
+    noise_seed: int = 0
+    noise_per_channel: bool = False
+    gradient_relative: bool = True
+    gradient_scale: float = 1.0
+    decay: float = 0.0
+    input_min_percentage: float = 0.95
+    noise_up: Optional[torch.Tensor] = None       # injected noise [n_tiles, T*k, F] (parity runs)
+    noise_down: Optional[torch.Tensor] = None
+
+
+class AnalogMoEFFN(torch.autograd.Function):
+    """y[t] = sum_j gate[t,j] * A(relu(A(x[t], keys[e_tj])), values[e_tj]).
+    input_range: [2, E, n_tiles] (row 0 up-, row 1 down-projection) or None."""
+
+    @staticmethod
+    def forward(ctx, x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
+        T, D = x.shape
+        E, _, F = keys.shape
+        k = sel_idx.shape[-1]
+        M = T * k
+        sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
+        ntu = 1 if cfg.bounds_up is None else len(cfg.bounds_up) - 1
+        ntd = 1 if cfg.bounds_down is None else len(cfg.bounds_down) - 1
+        ir_up = ir_dn = None
+        if input_range is not None:
+            ir3 = input_range.detach().float().reshape(2, E, -1)
+            ir_up, ir_dn = ir3[0, :, :ntu].contiguous(), ir3[1, :, :ntd].contiguous()
+        gen = cfg.noise_std > 0 and cfg.noise_up is None
+        wu = wd = None
+        if cfg.out_bound > 0 or gen:
+            wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
+            wd = ops.weight_abs_max(values, cfg.noise_per_channel)
+        common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
+                      noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
+        p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, bounds=cfg.bounds_up,
+                          noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True, **common)
+        z = ops.cvmm_fwd(p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn, bounds=cfg.bounds_down,
+                         noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd, **common)
+        y = ops.gate_reduce(z, gate)
+        ctx.save_for_backward(x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn)
+        ctx.cfg = cfg
+        ctx.ir_shape = None if input_range is None else input_range.shape
+        ctx.ir_dtype = None if input_range is None else input_range.dtype
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn = ctx.saved_tensors
+        cfg = ctx.cfg
+        E = keys.shape[0]
+        k = gate.shape[-1]
+        M = perm.numel()
+        dy = dy.contiguous()
+        by = dict(ir_by_expert=ir_up is not None)
+        irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
+                    input_min_percentage=cfg.input_min_percentage)
+        tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+        grad_values = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, bounds=cfg.bounds_down, g_scale=gate,
+                                     **by)
+        gp1, irg_dn = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate, ir=ir_dn,
+                                     bounds=cfg.bounds_down, relu_mask=True, **irkw, **by)
+        grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+        grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
+        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
+                                      bounds=cfg.bounds_up, **irkw, **by)
+        grad_x = ops.ksum(full, k) if k > 1 else full
+        grad_ir = None
+        if ir_up is not None and ctx.needs_input_grad[3]:
+            ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
+            gi = torch.zeros((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
+            gi[0, :, :ntu] = ops.segment_sum(irg_up, offsets, E)
+            gi[1, :, :ntd] = ops.segment_sum(irg_dn, offsets, E)
+            grad_ir = gi.reshape(ctx.ir_shape).to(ctx.ir_dtype)
+        return grad_x, grad_keys, grad_values, grad_ir, grad_gate, None, None

@@ -1,0 +1,404 @@
+"""SigmaMoE feed-forward layer (digital base) and its analog, hardware-aware version.
+
+``AnalogSigmaMoELayer`` keeps the constructor, the ``rpu_config`` API, the overridable hooks
+``compute_scores`` / ``cvmm_wrapper`` and the state-dict keys of the reference's
+``AnalogSigmaMoELayerAIHWKITLightning`` (analog_moe/moe_layer_aihwkit_lightning.py:134-570).
+Its base class there comes from the third-party ``sigma_moe`` package; ``SigmaMoELayer`` here
+restates the part of that contract the reference relies on (constructor keywords
+:261-276, attributes :220-233, forward = router -> top-k -> selection record ->
+compute_scores -> down-projection with gate reduction, as in the per-token form of
+test_moe_layer_aihwkit_lightning.py:82-107).
+
+Differences from the reference, all opt-in through ``rpu_config``: ``mapping.max_input_size``
+(K-tile split with one input range per tile), ``forward.out_bound`` / ``out_res`` (ADC) are
+implemented instead of asserted off (:152-160); output noise is drawn inside the kernel unless
+``noise_mode="injected"`` is chosen.  The router stays a digital ``nn.Linear``.
+"""
+from __future__ import annotations
+
+import math
+from functools import partial
+from typing import Callable, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from . import ops
+from .config import (TorchInferenceRPUConfig, WeightClipType, WeightModifierType, enum_name, kernel_inp_res)
+from .cvmm import CVMM, AnalogExt, CVMMSel, cvmm_prepare_sel2, cvmm_std
+from .ffn import AnalogMoEFFN, FFNConfig
+
+
+class MoEConifgError(Exception):
+    """Exceptions related to MoE configuration (name as in the reference)."""
+
+
+class _PerfectIO:
+    """io_params of a digital call: no abs-max scaling (cvmm.py:735-739)."""
+    is_perfect = True
+    noise_management = "NONE"
+
+
+def tile_bounds(K: int, max_input_size: int):
+    """Near-equal K-tiles of at most ``max_input_size`` features; None for a single tile."""
+    if max_input_size is None or max_input_size <= 0 or max_input_size >= K:
+        return None
+    n = -(-K // max_input_size)
+    base, rem = divmod(K, n)
+    b = [0]
+    for i in range(n):
+        b.append(b[-1] + base + (1 if i < rem else 0))
+    return b
+
+
+class SigmaMoELayer(nn.Module):
+    def __init__(self, d_model: int, n_experts: int, expert_size: int, k: int, dropout: float = 0.0,
+                 selection_mode: str = "sigmoid", activation_after_topk: bool = False,
+                 activation: Callable = F.relu, bias: bool = False, v_dim: Optional[int] = None,
+                 sinkhorn_n_iters: int = 3, expert_dropout: float = 0.0, traceable: bool = False):
+        super().__init__()
+        if traceable:
+            raise MoEConifgError("traceable=True (per-expert module lists on the CPU) is not part of this "
+                                 "GPU-only package")
+        if selection_mode not in ("sigmoid", "softmax"):
+            raise MoEConifgError(f"selection_mode {selection_mode!r} is not implemented")
+        self.k_dim = d_model
+        self.v_dim = v_dim if v_dim is not None else d_model
+        self.n_experts = n_experts
+        self.expert_size = expert_size
+        self.size = n_experts * expert_size
+        self.dropout = dropout
+        self.selection_mode = selection_mode
+        self.activation_after_topk = activation_after_topk
+        self.activation = activation
+        self.n_heads = k
+        self.sinkhorn_n_iters = sinkhorn_n_iters
+        self.expert_dropout = expert_dropout
+        self.traceable = traceable
+        self.keys = nn.Parameter(torch.empty(n_experts, self.k_dim, expert_size))
+        self.values = nn.Parameter(torch.empty(n_experts, expert_size, self.v_dim))
+        self.expert_sel = nn.Linear(self.k_dim, n_experts, bias=False)
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(n_experts, expert_size))
+            self.o_bias = nn.Parameter(torch.zeros(self.v_dim))
+        else:
+            self.bias = None
+            self.o_bias = None
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.keys, std=1.0 / math.sqrt(self.k_dim))
+        nn.init.normal_(self.values, std=1.0 / math.sqrt(self.expert_size))
+        nn.init.normal_(self.expert_sel.weight, std=1.0 / math.sqrt(self.k_dim))
+
+    # -- hooks the analog layer overrides ------------------------------------------------------
+    def cvmm_wrapper(self, inputs: Tensor, sel_indices: CVMMSel, weights: Tensor) -> Tensor:
+        return CVMM.apply(inputs, sel_indices.sel_index, sel_indices.sel, weights, -1.0, None,
+                          sel_indices.out_index, sel_indices.reduction_weight, None, None, _PerfectIO(),
+                          AnalogExt(offsets=sel_indices.offsets))
+
+    def compute_scores(self, inp: Tensor, index: CVMMSel, expert_scores: Optional[Tensor] = None) -> Tensor:
+        scores = self.cvmm_wrapper(inp, index, self.keys)
+        if self.bias is not None:
+            scores = scores + self.bias[index.raw_sel]
+        scores = self.activation(scores)
+        if expert_scores is not None:
+            scores = scores * expert_scores[..., None]
+        if self.dropout > 0:
+            scores = F.dropout(scores, self.dropout, training=self.training)
+        return scores
+
+    # -- router ------------------------------------------------------------------------------------
+    def select(self, x: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        """Gate values and expert ids [..., k] of the top-k experts, and the regularisation loss."""
+        logits = self.expert_sel(x)
+        reg_loss = x.new_zeros(())
+        if self.training:
+            logp = F.log_softmax(logits.float(), dim=-1).flatten(end_dim=-2)
+            mean_logp = torch.logsumexp(logp, dim=0) - math.log(logp.shape[0])
+            reg_loss = (mean_logp.exp() * mean_logp).sum()          # minus entropy of the mean usage
+        sel = logits if self.activation_after_topk else self._sel_activation(logits)
+        if self.training and self.expert_dropout > 0:
+            mask = torch.rand_like(sel) < self.expert_dropout
+            sel = sel.masked_fill(mask, float("-inf"))
+        sel_val, sel_idx = sel.topk(self.n_heads, dim=-1, sorted=False)
+        if self.activation_after_topk:
+            sel_val = self._sel_activation(sel_val)
+        return sel_val, sel_idx, reg_loss
+
+    def _sel_activation(self, t: Tensor) -> Tensor:
+        return torch.sigmoid(t) if self.selection_mode == "sigmoid" else F.softmax(t, dim=-1)
+
+    def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
+        """Expert feed-forward for a given routing decision (what follows the router in forward)."""
+        if not x.is_cuda:
+            raise MoEConifgError("MoE layer executed on CPU: this package runs on the GPU only "
+                                 "(moe_layer_aihwkit_lightning.py:395-400 raises the same way)")
+        sel_indices = cvmm_prepare_sel2(sel_idx, self.n_experts)
+        scores = self.compute_scores(x, sel_indices)
+        down = sel_indices.clone()
+        down.reduction_weight = sel_val
+        down.sel_index = sel_indices.out_index
+        down.out_index = None
+        out = self.cvmm_wrapper(scores, down, self.values)
+        if self.o_bias is not None:
+            out = out + self.o_bias
+        return out
+
+    def forward(self, x: Tensor) -> Tuple[Tensor, Tensor]:
+        sel_val, sel_idx, reg_loss = self.select(x)
+        return self.forward_selected(x, sel_val, sel_idx), reg_loss
+
+
+def load_state_dict_pre_hook(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+    """Accept checkpoints written by the traceable layout (per-expert ``keys.{i}.input_range``
+    entries, moe_layer_aihwkit_lightning.py:66-105) by folding them into ``input_range [2, E]``."""
+    import re
+    if prefix + "input_range" in state_dict:
+        return
+    pat = re.compile(rf"^{re.escape(prefix)}(keys|values)\.(\d+)\.input_range$")
+    found = {}
+    for key in list(state_dict):
+        m = pat.match(key)
+        if m:
+            found[(m.group(1), int(m.group(2)))] = state_dict[key]
+    if not found:
+        return
+    n = 1 + max(i for _, i in found)
+    state_dict[prefix + "input_range"] = torch.stack([
+        torch.cat([found[("keys", i)].reshape(1) for i in range(n)]),
+        torch.cat([found[("values", i)].reshape(1) for i in range(n)])])
+    idx_key = next((k for k in state_dict if re.match(
+        rf"^{re.escape(prefix)}(keys|values)\.\d+\.input_range_update_idx$", k)), None)
+    if idx_key is not None:
+        state_dict[prefix + "input_range_update_idx"] = state_dict[idx_key].reshape(())
+    for key in list(state_dict):
+        if re.match(rf"^{re.escape(prefix)}(keys|values)\.\d+\.(input_range|input_range_update_idx|x_min|x_max)$",
+                    key):
+            state_dict.pop(key)
+
+
+class AnalogSigmaMoELayer(SigmaMoELayer):
+    """Analog SigmaMoE layer; ``rpu_config`` first, then the digital layer's keywords
+    (moe_layer_aihwkit_lightning.py:135-138).  ``noise_mode``: "kernel" draws the output noise in
+    the GEMM epilogue from a counter-based generator; "injected" materialises ``randn`` tensors as
+    the reference does (:472-492) and hands them to the kernel."""
+
+    def __init__(self, rpu_config: Optional[TorchInferenceRPUConfig] = None, *args, noise_mode: str = "kernel",
+                 **kwargs):
+        super().__init__(*args, **kwargs)
+        self.rpu_config = TorchInferenceRPUConfig() if rpu_config is None else rpu_config
+        if noise_mode not in ("kernel", "injected"):
+            raise MoEConifgError("noise_mode must be 'kernel' or 'injected'")
+        self.noise_mode = noise_mode
+        self._noise_calls = 0
+        self._register_load_state_dict_pre_hook(load_state_dict_pre_hook)
+        mis = getattr(self.rpu_config.mapping, "max_input_size", -1)
+        self.bounds_up = tile_bounds(self.k_dim, mis)
+        self.bounds_down = tile_bounds(self.expert_size, mis)
+        self.n_tiles = max(1 if self.bounds_up is None else len(self.bounds_up) - 1,
+                           1 if self.bounds_down is None else len(self.bounds_down) - 1)
+        self.input_range = None
+        ir_params = self.rpu_config.pre_post.input_range
+        if ir_params.enable:
+            self.input_range_update_idx = nn.Parameter(torch.tensor(0.0), requires_grad=False)
+            shape = (2, self.n_experts) if self.n_tiles == 1 else (2, self.n_experts, self.n_tiles)
+            ir = torch.full(shape, float(ir_params.init_value))
+            if ir_params.learn_input_range:
+                self.input_range = nn.Parameter(ir)
+            else:
+                del self.input_range
+                self.register_buffer("input_range", ir)
+
+    # -- conversion ---------------------------------------------------------------------------------
+    @classmethod
+    def from_digital(cls, module: SigmaMoELayer, rpu_config: TorchInferenceRPUConfig) -> "AnalogSigmaMoELayer":
+        layer = cls(rpu_config=rpu_config, d_model=module.k_dim, n_experts=module.n_experts,
+                    expert_size=module.expert_size, k=module.n_heads, dropout=module.dropout,
+                    selection_mode=module.selection_mode, activation_after_topk=module.activation_after_topk,
+                    activation=module.activation, bias=module.bias is not None, v_dim=module.v_dim,
+                    sinkhorn_n_iters=module.sinkhorn_n_iters, expert_dropout=module.expert_dropout,
+                    traceable=module.traceable)
+        layer.set_weights(module.expert_sel, module.keys, module.values, module.bias, module.o_bias)
+        return layer.to(device=module.keys.device, dtype=module.keys.dtype)
+
+    @classmethod
+    def to_digital(cls, module: "AnalogSigmaMoELayer") -> SigmaMoELayer:
+        layer = SigmaMoELayer(d_model=module.k_dim, n_experts=module.n_experts, expert_size=module.expert_size,
+                              k=module.n_heads, dropout=module.dropout, selection_mode=module.selection_mode,
+                              activation_after_topk=module.activation_after_topk, activation=module.activation,
+                              bias=module.bias is not None, v_dim=module.v_dim,
+                              sinkhorn_n_iters=module.sinkhorn_n_iters, expert_dropout=module.expert_dropout)
+        layer.keys.data = module.keys.data.detach().clone()
+        layer.values.data = module.values.data.detach().clone()
+        layer.expert_sel.load_state_dict(module.expert_sel.state_dict())
+        if module.bias is not None:
+            layer.bias.data = module.bias.data.detach().clone()
+            layer.o_bias.data = module.o_bias.data.detach().clone()
+        return layer.to(device=module.keys.device, dtype=module.values.dtype)
+
+    def set_weights(self, expert_sel: nn.Linear, keys: Tensor, values: Tensor, bias: Optional[Tensor] = None,
+                    o_bias: Optional[Tensor] = None) -> None:
+        self.expert_sel.weight.data = expert_sel.weight.detach().clone()
+        if expert_sel.bias is not None and self.expert_sel.bias is not None:
+            self.expert_sel.bias.data = expert_sel.bias.detach().clone()
+        self.keys.data = keys.detach().clone()
+        self.values.data = values.detach().clone()
+        if bias is not None and self.bias is not None:
+            self.bias.data = bias.detach().clone()
+        if o_bias is not None and self.o_bias is not None:
+            self.o_bias.data = o_bias.detach().clone()
+
+    # -- weight modifier / clipping (moe_layer_aihwkit_lightning.py:313-382, 509-543) -----------------
+    @staticmethod
+    def modify_weight(inp_weight: Tensor, modifier) -> Tensor:
+        kind = enum_name(modifier.type)
+        if kind == "NONE":
+            return inp_weight
+        if kind.endswith("PER_CHANNEL"):
+            wmax = inp_weight.abs().amax(1, keepdim=True)
+        else:
+            wmax = inp_weight.reshape(inp_weight.size(0), -1).abs().amax(-1).view(-1, 1, 1)
+        if kind.startswith("DISCRETIZE"):
+            n_states = max(modifier.res, 1 / modifier.res)
+            res = wmax / n_states
+            q = torch.round(inp_weight / res) * res
+            inp_weight = inp_weight + (q - inp_weight).detach()        # straight-through quantiser
+        if "ADD_NORMAL" in kind:
+            with torch.no_grad():
+                noise = modifier.std_dev * wmax * torch.randn_like(inp_weight)
+            inp_weight = inp_weight + noise
+        return inp_weight
+
+    def post_update_step(self) -> None:
+        if hasattr(self.rpu_config, "clip") and enum_name(self.rpu_config.clip.type) != "NONE":
+            self.clip_weights()
+
+    @torch.no_grad()
+    def clip_weights(self) -> None:
+        kind = enum_name(self.rpu_config.clip.type)
+        if kind == "NONE":
+            return
+        sigma = self.rpu_config.clip.sigma
+        assert sigma > 0, "Clip sigma must be greater than 0"
+        if kind not in ("LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL"):
+            raise ValueError(f"Unknown clip type {self.rpu_config.clip.type}")
+        dims = (1, 2) if kind == "LAYER_GAUSSIAN" else 1
+        for w in (self.keys, self.values):
+            bound = sigma * w.std(dims, keepdim=True)
+            w.data = torch.minimum(torch.maximum(w.data, -bound), bound)
+
+    # -- the analog matmul ------------------------------------------------------------------------------
+    def _update_input_range_from_data(self, inputs: Tensor, sel_indices: CVMMSel, ir_idx: int) -> None:
+        """Running average of init_std_alpha * std during the first init_from_data calls; one counter
+        for both projections (moe_layer_aihwkit_lightning.py:432-445)."""
+        ir_params = self.rpu_config.pre_post.input_range
+        idx = self.input_range_update_idx
+        if not (idx < ir_params.init_from_data):
+            return
+        stds = cvmm_std(inputs, sel_indices.sel_index, sel_indices.sel, self.n_experts).float()
+        ok = stds > 0.0
+        if ok.any():
+            ir = self.input_range.data[ir_idx]
+            upd = (ir * idx + ir_params.init_std_alpha * (stds if ir.dim() == 1 else stds[:, None])) / (idx + 1)
+            ir[ok] = upd[ok].to(ir.dtype)
+            self.input_range_update_idx.data += 1
+        self.input_range.data = self.input_range.data.abs()
+
+    def _noise_seed(self) -> int:
+        self._noise_calls += 1
+        return (torch.initial_seed() * 0x9E3779B97F4A7C15 + self._noise_calls * 0xD1B54A32D192ED03) & (2 ** 63 - 1)
+
+    def cvmm_wrapper(self, inputs: Tensor, sel_indices: CVMMSel, weights: Tensor) -> Tensor:
+        """moe_layer_aihwkit_lightning.py:412-507."""
+        if not inputs.is_cuda:
+            raise MoEConifgError("Analog MoE executed on CPU. This package runs on the GPU only.")
+        fwd = self.rpu_config.forward
+        is_up = inputs.ndim == 3
+        ir_idx = 0 if is_up else 1
+        bounds = self.bounds_up if is_up else self.bounds_down
+        nt = 1 if bounds is None else len(bounds) - 1
+        bir = None
+        if self.input_range is not None:
+            if self.training:
+                self._update_input_range_from_data(inputs, sel_indices, ir_idx)
+            ir = self.input_range[ir_idx]
+            if ir.dim() == 2:
+                ir = ir[:, :nt]
+            bir = ir[sel_indices.sel]                                   # [..., k(, n_tiles)]
+        inp_res = kernel_inp_res(fwd.inp_res)
+        modified = weights
+        if (self.training or self.rpu_config.modifier.enable_during_test) and \
+                enum_name(self.rpu_config.modifier.type) != "NONE":
+            modified = self.modify_weight(weights.clone(), self.rpu_config.modifier)
+        ext = AnalogExt(offsets=sel_indices.offsets, bounds=bounds, out_bound=float(getattr(fwd, "out_bound", -1)),
+                        out_res=float(getattr(fwd, "out_res", -1)))
+        per_channel = bool(getattr(fwd, "out_noise_per_channel", False))
+        noisy = self.training and fwd.out_noise > 0
+        if ext.out_bound > 0 or noisy:
+            ext.wmax = ops.weight_abs_max(weights, per_channel)
+        out_noise = None
+        if noisy and self.noise_mode == "kernel":
+            ext.noise_std, ext.noise_seed = float(fwd.out_noise), self._noise_seed()
+        elif noisy:
+            shape = (nt, *sel_indices.raw_sel.shape, weights.shape[-1])
+            out_noise = torch.randn(shape, device=inputs.device) * fwd.out_noise * ext.wmax[sel_indices.raw_sel]
+        return CVMM.apply(inputs, sel_indices.sel_index, sel_indices.sel, modified, inp_res, bir,
+                          sel_indices.out_index, sel_indices.reduction_weight, out_noise,
+                          self.rpu_config.pre_post.input_range, fwd, ext)
+
+    # -- fused path ---------------------------------------------------------------------------------------
+    def _fusable(self) -> bool:
+        return (self.activation is F.relu and self.bias is None and self.dropout == 0 and
+                self.input_range is not None and enum_name(self.rpu_config.modifier.type) == "NONE" and
+                not (self.training and self.input_range_update_idx < self.rpu_config.pre_post.input_range.init_from_data))
+
+    def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
+        if not x.is_cuda or not self._fusable():
+            return super().forward_selected(x, sel_val, sel_idx)
+        fwd = self.rpu_config.forward
+        irp = self.rpu_config.pre_post.input_range
+        noisy = self.training and fwd.out_noise > 0
+        cfg = FFNConfig(inp_res=kernel_inp_res(fwd.inp_res), bounds_up=self.bounds_up, bounds_down=self.bounds_down,
+                        out_bound=float(getattr(fwd, "out_bound", -1)), out_res=float(getattr(fwd, "out_res", -1)),
+                        noise_std=float(fwd.out_noise) if noisy else 0.0, noise_seed=self._noise_seed() if noisy else 0,
+                        noise_per_channel=bool(getattr(fwd, "out_noise_per_channel", False)),
+                        gradient_relative=getattr(irp, "gradient_relative", True),
+                        gradient_scale=getattr(irp, "gradient_scale", 1.0), decay=irp.decay,
+                        input_min_percentage=irp.input_min_percentage)
+        if noisy and self.noise_mode == "injected":
+            E, k = self.n_experts, self.n_heads
+            M = sel_idx.numel()
+            flat = sel_idx.reshape(-1)
+            pc = cfg.noise_per_channel
+            wu, wd = ops.weight_abs_max(self.keys, pc), ops.weight_abs_max(self.values, pc)
+            ntu = 1 if self.bounds_up is None else len(self.bounds_up) - 1
+            ntd = 1 if self.bounds_down is None else len(self.bounds_down) - 1
+            cfg.noise_up = torch.randn(ntu, M, self.expert_size, device=x.device) * fwd.out_noise * wu[flat]
+            cfg.noise_down = torch.randn(ntd, M, self.v_dim, device=x.device) * fwd.out_noise * wd[flat]
+        lead = x.shape[:-1]
+        y = AnalogMoEFFN.apply(x.reshape(-1, x.shape[-1]), self.keys.to(x.dtype), self.values.to(x.dtype),
+                               self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
+                               sel_idx.reshape(-1, self.n_heads), cfg)
+        y = y.view(*lead, self.v_dim)
+        if self.o_bias is not None:
+            y = y + self.o_bias
+        return y
+
+    # -- checkpointing: the config travels with the state dict (:545-570) ------------------------------------
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        destination._metadata[prefix.split(".")[0]]["rpu_config"] = self.rpu_config
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+        if "rpu_config" in local_metadata:
+            self.rpu_config = local_metadata["rpu_config"]
+
+
+# Names under which the reference exports its two flavours (analog_moe/__init__.py).
+AnalogSigmaMoELayerAIHWKITLightning = AnalogSigmaMoELayer
+AnalogSigmaMoELayerAIHWKIT = AnalogSigmaMoELayer

@@ -94,8 +94,10 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
              ir: Optional[torch.Tensor] = None, abs_max: Optional[torch.Tensor] = None, inp_res: float = -1.0,
              bounds: Optional[Sequence[int]] = None, noise: Optional[torch.Tensor] = None,
              noise_std: float = 0.0, noise_seed: int = 0, wmax: Optional[torch.Tensor] = None,
-             out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False) -> torch.Tensor:
-    """out[out_index[i]] = analog(x[in_index[i]]) @ w[sel_sorted[i]] -> [n_out_rows, N]."""
+             out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
+             ir_by_expert: bool = False) -> torch.Tensor:
+    """out[out_index[i]] = analog(x[in_index[i]]) @ w[sel_sorted[i]] -> [n_out_rows, N].
+    ir: [M, n_tiles] per sorted position, or the [E, n_tiles] table with ir_by_expert."""
     _need_gpu(x, w, sel_sorted, offsets, in_index, out_index, ir, abs_max, noise, wmax)
     x2 = _rows2d(x)
     if w.stride(2) != 1 and w.stride(1) != 1:
@@ -103,17 +105,21 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
     out = torch.empty((n_out_rows, w.shape[2]), dtype=x2.dtype, device=x2.device)
     raw.cvmm_fwd(get_lib(), _stream(x2), x2, w, out, sel_sorted, offsets, in_index, out_index, _f32c(ir),
                  _f32c(abs_max), inp_res, bounds, _f32c(noise), noise_std, noise_seed, _f32c(wmax), out_bound,
-                 out_res, relu)
+                 out_res, relu, None, ir_by_expert)
     return out
 
 
 def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,
                g_index: Optional[torch.Tensor], *, ir: Optional[torch.Tensor] = None,
-               bounds: Optional[Sequence[int]] = None) -> torch.Tensor:
-    _need_gpu(x, g, offsets, in_index, g_index, ir)
+               bounds: Optional[Sequence[int]] = None, ir_by_expert: bool = False,
+               g_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """grad_w[e] = sum_i clamp(x[in_index[i]])^T (g_scale[in_index[i]] * g[g_index[i]])."""
+    _need_gpu(x, g, offsets, in_index, g_index, ir, g_scale)
     x2, g2 = _rows2d(x), _rows2d(g)
     grad_w = torch.empty((n_experts, x2.shape[1], g2.shape[1]), dtype=x2.dtype, device=x2.device)
-    raw.cvmm_bwd_w(get_lib(), _stream(x2), x2, g2, grad_w, offsets, in_index, g_index, _f32c(ir), bounds)
+    gs = None if g_scale is None else g_scale.detach().reshape(-1).to(x2.dtype).contiguous()
+    raw.cvmm_bwd_w(get_lib(), _stream(x2), x2, g2, grad_w, offsets, in_index, g_index, _f32c(ir), bounds,
+                   ir_by_expert, gs)
     return grad_w
 
 
@@ -122,7 +128,7 @@ def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index:
                xf_index: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
                ir: Optional[torch.Tensor] = None, bounds: Optional[Sequence[int]] = None,
                gradient_relative: bool = True, gradient_scale: float = 1.0, decay: float = 0.0,
-               input_min_percentage: float = 0.95, relu_mask: bool = False):
+               input_min_percentage: float = 0.95, relu_mask: bool = False, ir_by_expert: bool = False):
     """Returns (grad_x_full [n_out_rows, K], ir_grad [M, n_tiles] or None)."""
     _need_gpu(g, w, offsets, g_index, out_index, x, xf_index, gate, ir)
     lib = get_lib()
@@ -141,7 +147,8 @@ def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index:
         ws = torch.empty(max(raw.bwd_x_workspace_bytes(lib, M, K, n_tiles), 4), dtype=torch.uint8, device=g2.device)
     gate_c = None if gate is None else gate.detach().reshape(-1).to(g2.dtype).contiguous()
     raw.cvmm_bwd_x(lib, _stream(g2), g2, w, full, offsets, g_index, out_index, x2, xf_index, gate_c, ir32, ir_grad,
-                   bounds, gradient_relative, gradient_scale, decay, input_min_percentage, relu_mask, ws)
+                   bounds, gradient_relative, gradient_scale, decay, input_min_percentage, relu_mask, ws,
+                   ir_by_expert)
     return full, ir_grad
 
 

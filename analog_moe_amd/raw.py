@@ -66,7 +66,7 @@ def offsets_from_sorted(lib, stream, sel_sorted, E: int, offsets):
 def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=None, ir=None, abs_max=None,
              inp_res: float = -1.0, bounds: Optional[Sequence[int]] = None, noise=None, noise_std: float = 0.0,
              noise_seed: int = 0, wmax=None, out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
-             range_flag=None):
+             range_flag=None, ir_by_expert: bool = False):
     """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N]."""
     _rows(x, "x"); _rows(out, "out")
     a = FwdArgs()
@@ -85,8 +85,9 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
     a.sel_sorted, a.offsets = _p(_i32(sel_sorted, "sel_sorted")), _p(_i32(offsets, "offsets"))
     a.in_index, a.out_index = _p(_i32(in_index, "in_index")), _p(_i32(out_index, "out_index"))
     set_bounds(a, [0, K] if bounds is None else bounds)
-    if ir is not None and ir.numel() != M * a.n_tiles:
-        raise ValueError("ir must hold one value per sorted position and K-tile")
+    if ir is not None and ir.numel() != (E if ir_by_expert else M) * a.n_tiles:
+        raise ValueError("ir must hold one value per sorted position (or expert) and K-tile")
+    a.ir_by_expert = int(bool(ir_by_expert))
     a.ir, a.abs_max, a.inp_res = _p(_f32(ir, "ir")), _p(_f32(abs_max, "abs_max")), float(inp_res)
     if noise is not None:
         _f32(noise, "noise")
@@ -103,7 +104,7 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
 
 
 def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=None,
-               bounds: Optional[Sequence[int]] = None):
+               bounds: Optional[Sequence[int]] = None, ir_by_expert: bool = False, g_scale=None):
     """x [*, K]; g [*, N]; grad_w [E, K, N] contiguous."""
     _rows(x, "x"); _rows(g, "g")
     if not grad_w.is_contiguous():
@@ -120,7 +121,10 @@ def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=No
     a.offsets, a.in_index, a.g_index = _p(_i32(offsets, "offsets")), _p(_i32(in_index, "in_index")), \
         _p(_i32(g_index, "g_index"))
     set_bounds(a, [0, K] if bounds is None else bounds)
-    a.ir = _p(_f32(ir, "ir"))
+    a.ir, a.ir_by_expert = _p(_f32(ir, "ir")), int(bool(ir_by_expert))
+    if g_scale is not None and (g_scale.dtype != x.dtype or not g_scale.is_contiguous()):
+        raise TypeError("g_scale must be contiguous and share the dtype of x")
+    a.g_scale = _p(g_scale)
     check(lib, lib.amoe_cvmm_bwd_w(C.byref(a), stream), "amoe_cvmm_bwd_w")
 
 
@@ -131,7 +135,7 @@ def bwd_x_workspace_bytes(lib, M: int, K: int, n_tiles: int) -> int:
 def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=None, xf_index=None, gate=None,
                ir=None, ir_grad=None, bounds: Optional[Sequence[int]] = None, gradient_relative: bool = True,
                gradient_scale: float = 1.0, decay: float = 0.0, input_min_percentage: float = 0.95,
-               relu_mask: bool = False, workspace=None):
+               relu_mask: bool = False, workspace=None, ir_by_expert: bool = False):
     """g [*, N]; w [E, K, N] with N contiguous; grad_x_full [R_out, K]; x [*, K] forward input."""
     _rows(g, "g"); _rows(grad_x_full, "grad_x_full")
     a = BwdXArgs()
@@ -155,6 +159,7 @@ def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=No
     a.gate = _p(gate)
     set_bounds(a, [0, K] if bounds is None else bounds)
     a.ir, a.ir_grad = _p(_f32(ir, "ir")), _p(_f32(ir_grad, "ir_grad"))
+    a.ir_by_expert = int(bool(ir_by_expert))
     a.gradient_relative, a.gradient_scale = int(bool(gradient_relative)), float(gradient_scale)
     a.decay, a.input_min_percentage = float(decay), float(input_min_percentage)
     a.relu_mask = int(bool(relu_mask))

@@ -1,0 +1,201 @@
+"""Benchmark of the CVMM hot path: one analog SigmaMoE layer, forward + backward, on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input already resident in HBM:
+expert sort -> up-projection (DAC, K-tile split, noise, ADC, ReLU) -> down-projection ->
+gate-weighted reduction, then the full backward (both weight gradients, both input gradients
+with clip masks, input-range gradients, gate gradient).  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c2_f32|c4|c1]
+
+The default workload is BASELINE.json's 64-expert tile-split layer (configs[2]), the one its
+metric's MFMA-peak target is quoted on.  Only one GPU is used; --gpus N > 1 exits.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # T tokens, D d_model, E experts, F expert_size, k heads
+    "c1": dict(T=256, D=128, E=8, F=64, k=2, dtype="f32", routing="router", mis=-1, noise=0.0,
+               name="config1: d_model=128 E=8 F=64 k=2 256 tokens fp32"),
+    "c2": dict(T=8192, D=412, E=16, F=128, k=4, dtype="bf16", routing="router", mis=-1, noise=0.04,
+               name="config2: d_model=412 E=16 F=128 k=4 8192 tokens bf16"),
+    "c2_f32": dict(T=8192, D=412, E=16, F=128, k=4, dtype="f32", routing="router", mis=-1, noise=0.04,
+                   name="config2: d_model=412 E=16 F=128 k=4 8192 tokens fp32"),
+    "c3": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="bf16", routing="uniform", mis=512, noise=0.04,
+               name="config3: d_model=1024 (2x512 tiles) E=64 F=256 k=8 16384 tokens bf16 uniform routing"),
+    "c4": dict(T=32768, D=2048, E=128, F=512, k=4, dtype="bf16", routing="zipf", mis=-1, noise=0.04,
+               name="config4: d_model=2048 E=128 F=512 k=4 32768 tokens bf16 Zipf(1.2) routing"),
+}
+PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
+
+
+def cpu_baseline(cfg, pr, budget_tokens):
+    """Per-expert eager-PyTorch layer (oracle/layer_cpu.py) on the host cores, fp32, on the first
+    `budget_tokens` tokens of the same inputs; noise tensors are drawn inside the timed region."""
+    import torch
+    from oracle.layer_cpu import moe_layer_per_expert
+    from oracle.cvmm_oracle import tile_bounds
+    n = min(budget_tokens, cfg["T"])
+    E, k, D, F = cfg["E"], cfg["k"], cfg["D"], cfg["F"]
+    x = pr["x"][:n].float().cpu().requires_grad_()
+    keys = pr["keys"].float().cpu().requires_grad_()
+    values = pr["values"].float().cpu().requires_grad_()
+    gate = pr["gate"][:n].float().cpu().requires_grad_()
+    idx = pr["idx"][:n].cpu()
+    dy = pr["dy"][:n].float().cpu()
+    bu, bd = tile_bounds(D, cfg["mis"]), tile_bounds(F, cfg["mis"])
+    ir = torch.full((2, E, max(len(bu), len(bd)) - 1), 3.0, requires_grad=True)
+
+    def step():
+        wu = keys.detach().abs().amax((1, 2)).reshape(E, 1)
+        wd = values.detach().abs().amax((1, 2)).reshape(E, 1)
+        nu = nd = None
+        if cfg["noise"] > 0:
+            flat = idx.reshape(-1)
+            nu = torch.randn(len(bu) - 1, n * k, F) * cfg["noise"] * wu[flat]
+            nd = torch.randn(len(bd) - 1, n * k, D) * cfg["noise"] * wd[flat]
+        y = moe_layer_per_expert(x, keys, values, idx, gate, ir, inp_res=1 / 127, noise_up=nu, noise_down=nd,
+                                 wmax_up=wu, wmax_down=wd, out_bound=12.0, out_res=254.0, bounds_up=bu,
+                                 bounds_down=bd)
+        y.backward(dy)
+        for t in (x, keys, values, gate, ir):
+            t.grad = None
+
+    step()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t0 < 8.0 and reps < 20):
+        step()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": n / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {n} of {cfg['T']} tokens, all {E} experts, fp32, {reps} iterations, "
+                      f"{dt * 1e3:.1f} ms each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU hot path only; run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from analog_moe_amd import config as cfgmod, ops
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayer
+    from tests import util
+
+    cfg = CONFIGS[args.config]
+    ops.get_lib()
+    dev = torch.device("cuda:0")
+    tdt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    T, D, E, F, k = (cfg[n] for n in "TDEFk")
+
+    rpu = cfgmod.TorchInferenceRPUConfig()
+    rpu.forward.inp_res = 2 ** 8 - 2
+    rpu.forward.out_res = 2 ** 8 - 2
+    rpu.forward.out_bound = 12.0
+    rpu.forward.out_noise = cfg["noise"]
+    rpu.mapping.max_input_size = cfg["mis"]
+    rpu.pre_post.input_range.enable = True
+    rpu.pre_post.input_range.learn_input_range = True
+    rpu.pre_post.input_range.init_value = 3.0
+    rpu.pre_post.input_range.decay = 0.01
+    torch.manual_seed(0)
+    layer = AnalogSigmaMoELayer(rpu, d_model=D, n_experts=E, expert_size=F, k=k).to(dev).to(tdt)
+    layer.train()
+    pr = util.make_problem(0, T, D, E, F, k, dtype=tdt, routing=cfg["routing"])
+    with torch.no_grad():
+        layer.keys.copy_(pr["keys"])
+        layer.values.copy_(pr["values"])
+    x = pr["x"].to(dev).requires_grad_()
+    gate = pr["gate"].to(dev).requires_grad_()
+    idx = pr["idx"].to(dev)
+    dy = pr["dy"].to(dev)
+    params = [layer.keys, layer.values, layer.input_range, x, gate]
+
+    def step():
+        y = layer.forward_selected(x, gate, idx)
+        y.backward(dy)
+        for p in params:
+            p.grad = None
+
+    # HIP events around every launch of the GEMM kernels, on the stream they are launched on
+    events = {}
+
+    def timed(name):
+        fn = getattr(ops, name)
+
+        def wrapper(*a, **kw):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            r = fn(*a, **kw)
+            e.record()
+            events.setdefault(name, []).append((s, e))
+            return r
+        return fn, wrapper
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    saved = {}
+    for name in ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x", "prepare_sel", "gate_reduce", "gate_grad", "ksum",
+                 "weight_abs_max", "segment_sum"):
+        saved[name], w = timed(name)
+        setattr(ops, name, w)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for name, fn in saved.items():
+        setattr(ops, name, fn)
+
+    ms = elapsed / args.steps * 1e3
+    M = T * k
+    flops_step = 12.0 * M * D * F                 # six GEMM passes of 2*M*D*F
+    kern = {n: sum(s.elapsed_time(e) for s, e in ev) / len(ev) for n, ev in events.items()}
+    calls = {n: len(ev) // args.steps for n, ev in events.items()}
+    per_step = {n: kern[n] * calls[n] for n in kern}
+    gemms = ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x")
+    dom = max(gemms, key=lambda n: per_step[n])
+    gemm_flops = 2.0 * M * D * F                  # algorithmic flops of one launch of any of them
+    achieved = gemm_flops / (kern[dom] * 1e-3)
+    peak = PEAK[cfg["dtype"]]
+    out = {
+        "metric": "analog MoE layer fwd+bwd tokens/sec on 1 GPU; % of MFMA peak TFLOP/s",
+        "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": cfg["name"], "tokens": T, "d_model": D, "n_experts": E, "expert_size": F,
+                   "top_k": k, "analog": "learned input range 3.0, 8-bit DAC, 8-bit ADC (out_bound 12), "
+                   f"output noise {cfg['noise']} x max|W| drawn in-kernel, max_input_size {cfg['mis']}"},
+        "tflops": flops_step / (ms * 1e-3) / 1e12,
+        "pct_of_mfma_peak": 100.0 * flops_step / (ms * 1e-3) / peak,
+        "roofline": {"bound": "mfma", "kernel": {"cvmm_fwd": "gemm_rows_kernel (forward)",
+                                                  "cvmm_bwd_w": "gemm_wgrad_kernel",
+                                                  "cvmm_bwd_x": "gemm_rows_kernel (input gradient)"}[dom],
+                     "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
+                     "frac": achieved / peak, "traffic": None,
+                     "flops_per_launch": gemm_flops, "avg_launch_ms": kern[dom]},
+        "kernel_ms_per_step": {n: round(v, 4) for n, v in sorted(per_step.items(), key=lambda kv: -kv[1])},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, pr, args.cpu_tokens)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -85,6 +85,9 @@ typedef struct amoe_fwd_args {
   const int32_t* in_index;       /* [M] */
   const int32_t* out_index;      /* [M] or NULL -> in_index (cvmm.py:196-205) */
   const float* ir;               /* [M, n_tiles] input range per sorted position, or NULL */
+  int32_t ir_by_expert;          /* != 0: ir is the [E, n_tiles] table itself (what the caller
+                                    would otherwise gather with input_range[sel],
+                                    moe_layer_aihwkit_lightning.py:447-448) */
   const float* abs_max;          /* [n_in_rows] or NULL (cvmm.py:124-128, 156-158) */
   float inp_res;                 /* quantisation step; <= 0: no quantisation */
   int32_t n_tiles;               /* >= 1 */
@@ -122,6 +125,11 @@ typedef struct amoe_bwd_w_args {
   const int32_t* g_index;                /* [M] row of g per sorted position, NULL -> in_index
                                             (cvmm.py:346-351) */
   const float* ir;                       /* [M, n_tiles] or NULL */
+  int32_t ir_by_expert;                  /* != 0: ir is [E, n_tiles] */
+  const void* g_scale;                   /* dtype, indexed by in_index[i], or NULL: the g row is
+                                            multiplied by it and rounded to dtype, which is the
+                                            gate (x) dy outer product of cvmm.py:785-789 without
+                                            materialising it */
   int32_t n_tiles;
   int32_t tile_bounds[AMOE_MAX_TILES + 1];
 } amoe_bwd_w_args;
@@ -153,6 +161,7 @@ typedef struct amoe_bwd_x_args {
   const int32_t* xf_index;       /* [M] row of x */
   const void* gate;              /* [n_out_rows] dtype, indexed by output row, or NULL */
   const float* ir;               /* [M, n_tiles] or NULL */
+  int32_t ir_by_expert;          /* != 0: ir is [E, n_tiles]; ir_grad stays per sorted position */
   float* ir_grad;                /* [M, n_tiles] out (required when ir != NULL) */
   int32_t n_tiles;
   int32_t tile_bounds[AMOE_MAX_TILES + 1];

@@ -69,6 +69,9 @@ CASES = {
 def test_layer_parity_emulated(emu_ops, name):
     pk, lk, dtype, tol = CASES[name]
     lk = dict(lk)
+    # alternate between the per-position input-range vector of the reference and the fused
+    # per-expert table / in-kernel gate (x) dy product
+    lk["by_expert"] = list(CASES).index(name) % 2 == 1
     tdt = torch.float32 if dtype == "f32" else torch.bfloat16
     pr = util.make_problem(7, dtype=tdt, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
@@ -77,7 +80,7 @@ def test_layer_parity_emulated(emu_ops, name):
         nt = max(len(lk.get("bounds_up", [0, 1])), len(lk.get("bounds_down", [0, 1]))) - 1
         ir = torch.from_numpy(np.random.default_rng(1).uniform(0.7, 2.5, size=(2, E, nt)).astype(np.float32))
     nstd = lk.pop("noise", 0.0)
-    okw = dict(lk)
+    okw = {n: v for n, v in lk.items() if n != "by_expert"}
     if nstd:
         ntu = len(lk.get("bounds_up", [0, 1])) - 1
         ntd = len(lk.get("bounds_down", [0, 1])) - 1

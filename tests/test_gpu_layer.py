@@ -1,0 +1,156 @@
+"""GPU tests of the layer classes: AnalogSigmaMoELayer (fused path and the CVMM.apply
+composition of the reference) against the oracle; CVMM.apply against torch autograd with the
+analog features off; input-range initialisation from data."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cvmm_oracle as O
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(cfgmod, mods, d=128, E=4, F=64, k=2, dtype=torch.float32, **rpu_kw):
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayer
+    r = cfgmod.TorchInferenceRPUConfig()
+    r.forward.inp_res = rpu_kw.get("inp_res", 2 ** 8 - 2)
+    r.forward.out_noise = rpu_kw.get("out_noise", 0.0)
+    r.forward.out_bound = rpu_kw.get("out_bound", -1)
+    r.forward.out_res = rpu_kw.get("out_res", -1)
+    r.mapping.max_input_size = rpu_kw.get("max_input_size", -1)
+    ir = r.pre_post.input_range
+    ir.enable, ir.learn_input_range, ir.init_value = rpu_kw.get("ir", True), True, 2.0
+    ir.decay, ir.input_min_percentage = rpu_kw.get("decay", 0.0), 0.5
+    ir.init_from_data = rpu_kw.get("init_from_data", 0)
+    torch.manual_seed(0)
+    return AnalogSigmaMoELayer(r, d_model=d, n_experts=E, expert_size=F, k=k, **mods).cuda().to(dtype)
+
+
+def _oracle_for(layer, x, sel_val, sel_idx, dy, **kw):
+    ir = None if layer.input_range is None else layer.input_range.detach().float().cpu().numpy().reshape(
+        2, layer.n_experts, -1)
+    return O.layer_fwd_bwd(util.np32(x.reshape(-1, x.shape[-1])), util.np32(layer.keys), util.np32(layer.values),
+                           sel_idx.reshape(-1, layer.n_heads).cpu().numpy(),
+                           util.np32(sel_val.reshape(-1, layer.n_heads)), ir,
+                           util.np32(dy.reshape(-1, dy.shape[-1])), **kw)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("split", [False, True])
+def test_layer_matches_oracle(fused, split):
+    """Shapes of the reference's gradient test (test_moe_layer_aihwkit_lightning.py:211-217)."""
+    from analog_moe_amd import config as cfgmod
+    mods = {} if fused else {"dropout": 0.0, "bias": True}      # a bias switches the fused path off
+    layer = _layer(cfgmod, mods, decay=0.01, max_input_size=64 if split else -1)
+    assert layer._fusable() == fused
+    with torch.no_grad():
+        layer.input_range.copy_(torch.rand_like(layer.input_range) + 1.0)
+    x = torch.randn(10, 10, 128, device="cuda", requires_grad=True)
+    sel_val, sel_idx, _ = layer.select(x.detach())
+    sel_val = sel_val.detach().requires_grad_()
+    y = layer.forward_selected(x, sel_val, sel_idx)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    want = _oracle_for(layer, x, sel_val, sel_idx, dy, inp_res=1 / 127, decay=0.01, input_min_percentage=0.5,
+                       bounds_up=layer.bounds_up, bounds_down=layer.bounds_down)
+    tol = 1e-5
+    assert util.rel_err(util.np32(y).reshape(100, 128), want.y) < tol
+    assert util.rel_err(util.np32(x.grad).reshape(100, 128), want.grad_x) < tol
+    assert util.rel_err(util.np32(layer.keys.grad), want.grad_keys) < tol
+    assert util.rel_err(util.np32(layer.values.grad), want.grad_values) < tol
+    assert util.rel_err(util.np32(sel_val.grad).reshape(100, 2), want.grad_gate) < tol
+    assert util.rel_err(util.np32(layer.input_range.grad).reshape(want.grad_ir.shape), want.grad_ir) < 1e-4
+    if not fused:
+        assert layer.bias.grad is not None
+
+
+def test_full_forward_runs_router_and_returns_reg_loss():
+    from analog_moe_amd import config as cfgmod
+    layer = _layer(cfgmod, {}, dtype=torch.bfloat16, out_noise=0.04, out_bound=12.0, out_res=254.0)
+    layer.train()
+    x = torch.randn(4, 16, 128, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    y, reg = layer(x)
+    (y.float().sum() + reg).backward()
+    assert y.shape == x.shape and torch.isfinite(y).all() and torch.isfinite(x.grad).all()
+    assert layer.input_range.grad is not None and layer.expert_sel.weight.grad is not None
+    y2, _ = layer(x)
+    assert not torch.equal(y, y2)                      # a fresh noise draw per call
+    layer.eval()
+    a, _ = layer(x)
+    b, _ = layer(x)
+    assert torch.equal(a, b)                           # no noise at inference
+
+
+def test_injected_noise_mode_statistics():
+    """The reference's own noise check is statistical (tests/test_moe_layer_aihwkit.py:112-177): the
+    error's spread must match the configured noise level in both noise modes."""
+    from analog_moe_amd import config as cfgmod
+    stds = {}
+    for mode in ("kernel", "injected"):
+        layer = _layer(cfgmod, {"noise_mode": mode}, d=512, E=4, F=512, k=2, out_noise=0.05, inp_res=-1)
+        with torch.no_grad():
+            layer.input_range.fill_(100.0)
+        x = torch.randn(20, 50, 512, device="cuda")
+        sel_val, sel_idx, _ = layer.select(x)
+        layer.eval()
+        clean = layer.forward_selected(x, sel_val, sel_idx)
+        layer.train()
+        noisy = layer.forward_selected(x, sel_val, sel_idx)
+        stds[mode] = (noisy - clean).std(-1).mean().item()
+    assert stds["kernel"] == pytest.approx(stds["injected"], rel=0.05)
+
+
+def test_cvmm_apply_digital_matches_torch_autograd():
+    """Analog features off: CVMM.apply is a per-expert matmul; autograd of a plain torch
+    formulation gives the reference gradients (cvmm.py:699-897 with everything None)."""
+    from analog_moe_amd.cvmm import CVMM, cvmm_prepare_sel, cvmm_prepare_sel2
+    torch.manual_seed(1)
+    T, D, F, E, k = 64, 72, 40, 5, 2
+    x = torch.randn(T, 1, D, device="cuda", requires_grad=True)
+    keys = (torch.randn(E, D, F, device="cuda") / D ** 0.5).requires_grad_()
+    idx = torch.randint(0, E, (T, 1, k), device="cuda")
+    s = cvmm_prepare_sel2(idx, E)
+    io = type("IO", (), {"is_perfect": True, "noise_management": "NONE"})()
+    out = CVMM.apply(x, s.sel_index, s.sel, keys, -1.0, None, s.out_index, None, None, None, io)
+    assert out.shape == (T, 1, k, F)
+    g = torch.randn_like(out)
+    out.backward(g)
+    x2 = x.detach().clone().requires_grad_(); k2 = keys.detach().clone().requires_grad_()
+    ref = torch.einsum("td,tkdf->tkf", x2[:, 0], k2[idx[:, 0]]).view(T, 1, k, F)
+    ref.backward(g)
+    assert util.rel_err(util.np32(out), util.np32(ref)) < 1e-5
+    assert util.rel_err(util.np32(x.grad), util.np32(x2.grad)) < 1e-5
+    assert util.rel_err(util.np32(keys.grad), util.np32(k2.grad)) < 1e-5
+    # k = 1 record of the reference's cvmm_prepare_sel: sel_index is the permutation itself
+    s1 = cvmm_prepare_sel(idx[..., 0], E)
+    ssel, perm = torch.sort(idx[..., 0].flatten(), stable=True)
+    assert torch.equal(s1.sel_index.long(), perm) and torch.equal(s1.sel.flatten().long(), ssel)
+
+
+def test_abs_max_path_of_lightning_flavour():
+    """Input ranges disabled -> per-row abs-max scaling (cvmm.py:729-733); scale-equivariant."""
+    from analog_moe_amd import config as cfgmod
+    layer = _layer(cfgmod, {}, ir=False)
+    assert layer.input_range is None and not layer._fusable()
+    x = torch.randn(6, 7, 128, device="cuda")
+    sel_val, sel_idx, _ = layer.select(x)
+    a = layer.forward_selected(x, sel_val, sel_idx)
+    b = layer.forward_selected(4 * x, sel_val, sel_idx)
+    assert torch.allclose(4 * a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_input_range_init_from_data():
+    """moe_layer_aihwkit_lightning.py:432-445: running mean of init_std_alpha * std, one shared counter."""
+    from analog_moe_amd import config as cfgmod
+    layer = _layer(cfgmod, {}, init_from_data=4)
+    layer.train()
+    x = torch.randn(8, 32, 128, device="cuda")
+    sel_val, sel_idx, _ = layer.select(x)
+    layer.forward_selected(x, sel_val, sel_idx)
+    assert float(layer.input_range_update_idx) == 2.0            # up- and down-projection each advance it
+    flat = sel_idx.reshape(-1, 2).cpu().numpy()
+    s = O.prepare_sel(flat, 4, 2)
+    std_up = O.expert_std(util.np32(x.reshape(-1, 128)), s.in_index, s.sel_sorted, 4)
+    want_up = (2.0 * 0 + 3.0 * std_up) / 1                        # idx = 0 at the first call
+    np.testing.assert_allclose(layer.input_range.data[0].cpu().numpy(), want_up, rtol=1e-4)

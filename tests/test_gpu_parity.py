@@ -45,8 +45,8 @@ def test_prepare_sel_bit_exact(ops, M, E, k, skew):
     assert np.array_equal(got32[1].cpu().numpy(), want.perm)
 
 
-def _run_case(ops, pk, lk, dtype, seed=7, routing="router"):
-    lk = dict(lk)
+def _run_case(ops, pk, lk, dtype, seed=7, routing="router", by_expert=False):
+    lk = dict(lk, by_expert=by_expert)
     tdt = torch.float32 if dtype == "f32" else torch.bfloat16
     pr = util.make_problem(seed, dtype=tdt, routing=routing, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
@@ -59,7 +59,7 @@ def _run_case(ops, pk, lk, dtype, seed=7, routing="router"):
         else:
             ir = torch.full((2, E, nt), float(irspec))
     nstd = lk.pop("noise", 0.0)
-    okw = dict(lk)
+    okw = {n: v for n, v in lk.items() if n != "by_expert"}
     if nstd:
         ntu = len(lk.get("bounds_up", [0, 1])) - 1
         ntd = len(lk.get("bounds_down", [0, 1])) - 1
@@ -83,7 +83,7 @@ def _run_case(ops, pk, lk, dtype, seed=7, routing="router"):
 def test_layer_parity_small(ops, name):
     pk, lk, dtype, _ = CASES[name]
     print("case", name, flush=True)
-    print(_run_case(ops, pk, lk, dtype))
+    print(_run_case(ops, pk, lk, dtype, by_expert=list(CASES).index(name) % 2 == 1))
 
 
 def test_config1_cpu_runnable_layer(ops):
@@ -102,7 +102,7 @@ def test_config2_paper_scale_layer(ops, dtype):
     print("config 2", dtype, flush=True)
     errs = _run_case(ops, dict(T=8192, D=412, E=16, F=128, k=4),
                      dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01,
-                          input_min_percentage=0.9), dtype, seed=0)
+                          input_min_percentage=0.9), dtype, seed=0, by_expert=(dtype == "bf16"))
     print(errs)
 
 

@@ -37,7 +37,7 @@ def np32(t):
 def layer_ops_fwd_bwd(ops, pr, ir=None, *, inp_res=-1.0, noise_up=None, noise_down=None, noise_std=0.0,
                       noise_seed=None, out_bound=-1.0, out_res=-1.0, bounds_up=None, bounds_down=None, decay=0.0,
                       input_min_percentage=0.95, gradient_relative=True, gradient_scale=1.0, per_channel=False,
-                      backward=True):
+                      backward=True, by_expert=False):
     """The layer of oracle.layer_fwd_bwd, through the kernels.  ir [2, E, n_tiles] tensor or None."""
     x, keys, values, idx, gate, dy = (pr[n] for n in ("x", "keys", "values", "idx", "gate", "dy"))
     T, D = x.shape
@@ -49,19 +49,22 @@ def layer_ops_fwd_bwd(ops, pr, ir=None, *, inp_res=-1.0, noise_up=None, noise_do
     ntu = 1 if bounds_up is None else len(bounds_up) - 1
     ntd = 1 if bounds_down is None else len(bounds_down) - 1
     ir_up = ir_dn = None
-    if ir is not None:
+    if ir is not None and by_expert:
+        ir_up, ir_dn = ir[0][:, :ntu].contiguous(), ir[1][:, :ntd].contiguous()
+    elif ir is not None:
         ir_up = ir[0][sel_l][:, :ntu].contiguous()
         ir_dn = ir[1][sel_l][:, :ntd].contiguous()
+    be = dict(ir_by_expert=by_expert and ir is not None)
     need_wmax = out_bound > 0 or (noise_seed is not None and noise_std > 0)
     wu = ops.weight_abs_max(keys, per_channel) if need_wmax else None
     wd = ops.weight_abs_max(values, per_channel) if need_wmax else None
     gen = noise_seed is not None and noise_std > 0
     p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, inp_res=inp_res, bounds=bounds_up,
                       noise=noise_up, noise_std=noise_std if gen else 0.0, noise_seed=noise_seed or 0, wmax=wu,
-                      out_bound=out_bound, out_res=out_res, relu=True)
+                      out_bound=out_bound, out_res=out_res, relu=True, **be)
     z = ops.cvmm_fwd(p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn, inp_res=inp_res, bounds=bounds_down,
                      noise=noise_down, noise_std=noise_std if gen else 0.0, noise_seed=(noise_seed or 0) + 1,
-                     wmax=wd, out_bound=out_bound, out_res=out_res)
+                     wmax=wd, out_bound=out_bound, out_res=out_res, **be)
     y = ops.gate_reduce(z, gate)
     res = dict(y=y, scores=p1, z=z, sel_sorted=sel_sorted, perm=perm, in_index=in_index, offsets=offsets)
     if not backward:
@@ -69,16 +72,20 @@ def layer_ops_fwd_bwd(ops, pr, ir=None, *, inp_res=-1.0, noise_up=None, noise_do
     irkw = dict(gradient_relative=gradient_relative, gradient_scale=gradient_scale, decay=decay,
                 input_min_percentage=input_min_percentage)
     # down-projection backward (cvmm.py:785-889)
-    g_w = (gate.reshape(-1, 1) * dy.repeat_interleave(k, dim=0)).to(dy.dtype)
-    res["grad_values"] = ops.cvmm_bwd_w(p1, g_w, E, offsets, perm, None, ir=ir_dn, bounds=bounds_down)
     g_tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+    if by_expert:   # gate (x) dy formed inside the kernel
+        res["grad_values"] = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, g_tok, ir=ir_dn, bounds=bounds_down,
+                                            g_scale=gate, **be)
+    else:
+        g_w = (gate.reshape(-1, 1) * dy.repeat_interleave(k, dim=0)).to(dy.dtype)
+        res["grad_values"] = ops.cvmm_bwd_w(p1, g_w, E, offsets, perm, None, ir=ir_dn, bounds=bounds_down)
     gp1, irg_dn = ops.cvmm_bwd_x(dy, values, offsets, g_tok, perm, M, x=p1, xf_index=perm, gate=gate, ir=ir_dn,
-                                 bounds=bounds_down, relu_mask=True, **irkw)
+                                 bounds=bounds_down, relu_mask=True, **irkw, **be)
     res["grad_gate"] = ops.gate_grad(z, dy, k)
     # up-projection backward
-    res["grad_keys"] = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=bounds_up)
+    res["grad_keys"] = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=bounds_up, **be)
     full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
-                                  bounds=bounds_up, **irkw)
+                                  bounds=bounds_up, **irkw, **be)
     res["grad_x"] = ops.ksum(full, k)
     res["grad_p1"] = gp1
     if ir is not None:
