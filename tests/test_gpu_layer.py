@@ -38,11 +38,15 @@ def _oracle_for(layer, x, sel_val, sel_idx, dy, **kw):
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("split", [False, True])
-def test_layer_matches_oracle(fused, split):
-    """Shapes of the reference's gradient test (test_moe_layer_aihwkit_lightning.py:211-217)."""
+@pytest.mark.parametrize("quant", [False, True])
+def test_layer_matches_oracle(fused, split, quant):
+    """Shapes of the reference's gradient test (test_moe_layer_aihwkit_lightning.py:211-217).  Like that
+    test (:256-257, rounding switched off) the strict comparison runs without input quantisation: with
+    it, a last-bit difference in the up-projection can move a down-projection input across a rounding
+    boundary, which changes that product by one code step; the quantised runs get a tolerance for that."""
     from analog_moe_amd import config as cfgmod
     mods = {} if fused else {"dropout": 0.0, "bias": True}      # a bias switches the fused path off
-    layer = _layer(cfgmod, mods, decay=0.01, max_input_size=64 if split else -1)
+    layer = _layer(cfgmod, mods, decay=0.01, max_input_size=64 if split else -1, inp_res=254 if quant else -1)
     assert layer._fusable() == fused
     with torch.no_grad():
         layer.input_range.copy_(torch.rand_like(layer.input_range) + 1.0)
@@ -52,15 +56,15 @@ def test_layer_matches_oracle(fused, split):
     y = layer.forward_selected(x, sel_val, sel_idx)
     dy = torch.randn_like(y)
     y.backward(dy)
-    want = _oracle_for(layer, x, sel_val, sel_idx, dy, inp_res=1 / 127, decay=0.01, input_min_percentage=0.5,
-                       bounds_up=layer.bounds_up, bounds_down=layer.bounds_down)
-    tol = 1e-5
+    want = _oracle_for(layer, x, sel_val, sel_idx, dy, inp_res=1 / 127 if quant else -1, decay=0.01,
+                       input_min_percentage=0.5, bounds_up=layer.bounds_up, bounds_down=layer.bounds_down)
+    tol = 5e-3 if quant else 1e-5
     assert util.rel_err(util.np32(y).reshape(100, 128), want.y) < tol
     assert util.rel_err(util.np32(x.grad).reshape(100, 128), want.grad_x) < tol
     assert util.rel_err(util.np32(layer.keys.grad), want.grad_keys) < tol
     assert util.rel_err(util.np32(layer.values.grad), want.grad_values) < tol
     assert util.rel_err(util.np32(sel_val.grad).reshape(100, 2), want.grad_gate) < tol
-    assert util.rel_err(util.np32(layer.input_range.grad).reshape(want.grad_ir.shape), want.grad_ir) < 1e-4
+    assert util.rel_err(util.np32(layer.input_range.grad).reshape(want.grad_ir.shape), want.grad_ir) < max(tol, 1e-4)
     if not fused:
         assert layer.bias.grad is not None
 
