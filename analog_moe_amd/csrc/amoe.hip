@@ -365,12 +365,18 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
   if (!aligned(w, esize(dtype)) || !aligned(wmax, 4)) return AMOE_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (cols == 1 || N == 1) {
+    const long long per = (long long)K * N;
+    int chunks = (int)((per + 16 * kThreads - 1) / (16 * kThreads));
+    chunks = chunks < 1 ? 1 : (chunks > 64 ? 64 : chunks);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
+                       reinterpret_cast<uint32_t*>(wmax), (int)E);
+    if (int rc = launch_rc()) return rc;
     if (dtype == AMOE_F32) {
       auto kf = &weight_abs_max_kernel<float>;
-      hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const float*>(w), (long long)K * N, wmax);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax);
     } else {
       auto kf = &weight_abs_max_kernel<uint16_t>;
-      hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (long long)K * N, wmax);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax);
     }
   } else {
     dim3 grid((N + kThreads - 1) / kThreads, E);

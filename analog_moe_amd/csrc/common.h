@@ -43,61 +43,85 @@ template <> struct Elem<uint16_t> {    // bf16 bits
   static constexpr int kBK = 64;
   static constexpr int kMmaK = 16;
   static constexpr int kPadKC = 8;
-  static constexpr int kPadRC = 16;
+  static constexpr int kPadRC = 32;     // row stride 320 B: the four rows x two 16-column groups of a
+                                       // transposing read land on disjoint LDS banks
   static __device__ __forceinline__ float load(const uint16_t* p) { return bf16_to_f32(*p); }
   static __device__ __forceinline__ uint16_t cvt(float v) { return f32_to_bf16(v); }
   static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_to_f32(v); }
 };
 
-// 16 bytes of elements held as fp32 values in registers.
-template <typename T> struct Chunk { float v[Elem<T>::kChunk]; };
+// ---- 16-byte chunks --------------------------------------------------------------------------
+// Operands travel global -> registers -> LDS as raw 16-byte chunks; only the gathered rows of
+// the analog forward are unpacked to fp32 (for the DAC stage) on the way.
+typedef u32x4 Raw;
 
-template <typename T>
-__device__ __forceinline__ Chunk<T> chunk_zero() {
-  Chunk<T> c;
-#pragma unroll
-  for (int j = 0; j < Elem<T>::kChunk; j++) c.v[j] = 0.f;
-  return c;
-}
+__device__ __forceinline__ Raw raw_zero() { return Raw{0u, 0u, 0u, 0u}; }
 
 // Load one chunk starting at p (elements [0, n_valid) exist; the rest read as zero).
 // vec: p is 16-byte aligned and the caller allows vector access.
 template <typename T>
-__device__ __forceinline__ Chunk<T> chunk_load(const T* p, int n_valid, bool vec) {
+__device__ __forceinline__ Raw raw_load(const T* p, int n_valid, bool vec) {
   constexpr int C = Elem<T>::kChunk;
-  Chunk<T> c;
-  if (vec && n_valid >= C) {
-    u32x4 raw = *reinterpret_cast<const u32x4*>(p);
-    if constexpr (sizeof(T) == 4) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) c.v[j] = as_f32(raw[j]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        c.v[2 * j] = as_f32(raw[j] << 16);
-        c.v[2 * j + 1] = as_f32(raw[j] & 0xffff0000u);
-      }
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < C; j++) c.v[j] = (j < n_valid) ? Elem<T>::load(p + j) : 0.f;
-  }
-  return c;
-}
-
-// Store one chunk of fp32 values as T into LDS (always 16-byte aligned there).
-template <typename T>
-__device__ __forceinline__ void chunk_store_lds(T* p, const Chunk<T>& c) {
-  u32x4 raw;
+  if (vec && n_valid >= C) return *reinterpret_cast<const Raw*>(p);
+  Raw r = raw_zero();
+  if (n_valid <= 0) return r;
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) raw[j] = as_u32(c.v[j]);
+    for (int j = 0; j < 4; j++) r[j] = (j < n_valid) ? as_u32(p[j]) : 0u;
   } else {
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-      raw[j] = (uint32_t)f32_to_bf16(c.v[2 * j]) | ((uint32_t)f32_to_bf16(c.v[2 * j + 1]) << 16);
+    for (int j = 0; j < 4; j++) {
+      const uint32_t lo = (2 * j < n_valid) ? (uint32_t)p[2 * j] : 0u;
+      const uint32_t hi = (2 * j + 1 < n_valid) ? (uint32_t)p[2 * j + 1] : 0u;
+      r[j] = lo | (hi << 16);
+    }
   }
-  *reinterpret_cast<u32x4*>(p) = raw;
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void raw_unpack(const Raw& r, float (&v)[Elem<T>::kChunk]) {
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = as_f32(r[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j] = as_f32(r[j] << 16);
+      v[2 * j + 1] = as_f32(r[j] & 0xffff0000u);
+    }
+  }
+}
+
+// fp32 -> T with round to nearest even.
+template <typename T>
+__device__ __forceinline__ Raw raw_pack(const float (&v)[Elem<T>::kChunk]) {
+  Raw r;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) r[j] = as_u32(v[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++) r[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
+  }
+  return r;
+}
+
+// fp32 values that are exactly representable in bf16 (small integers): plain truncation.
+__device__ __forceinline__ Raw raw_pack_exact_bf16(const float (&v)[8]) {
+  Raw r;
+#pragma unroll
+  for (int j = 0; j < 4; j++) r[j] = (as_u32(v[2 * j]) >> 16) | (as_u32(v[2 * j + 1]) & 0xffff0000u);
+  return r;
+}
+
+// a / b given y = 1/b (correctly rounded): one multiply and two fused multiply-adds give the
+// correctly rounded quotient (checked against IEEE division over 4e8 random operand pairs of
+// the DAC stage's value ranges, including all-ones and near-power-of-two divisors).
+__device__ __forceinline__ float div_by(float a, float b, float y) {
+  const float q0 = a * y;
+  const float r = fmaf(-q0, b, a);
+  return fmaf(r, y, q0);
 }
 
 // Store 4 consecutive fp32 values as T to global memory at p; n_valid of them exist.

@@ -42,18 +42,27 @@ struct RowsParams {
   int a_vec, w_vec, out_vec, noise_vec, xf_vec;
 };
 
+// Workgroups are handed to the 8 XCDs round-robin; this maps the hardware id to a logical id so
+// that each XCD (one L2) works on a contiguous range of logical tiles.
+__device__ __forceinline__ int xcd_contiguous_id(int b, int grid) {
+  const int q = grid >> 3, r = grid & 7;
+  const int xcd = b & 7, idx = b >> 3;
+  return xcd * q + (xcd < r ? xcd : r) + idx;
+}
+
 template <typename T, bool W_KC, int MODE>
-__global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p) {
+__global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams p) {
   using EL = Elem<T>;
   constexpr int BK = EL::kBK, CH = EL::kChunk, MMAK = EL::kMmaK;
   constexpr int LDA = BK + EL::kPadKC;
   constexpr int LDB = W_KC ? (BK + EL::kPadKC) : (kTileCols + EL::kPadRC);
+  constexpr int A_ELEMS = kTileRows * LDA;
   constexpr int B_ELEMS = W_KC ? kTileCols * LDB : BK * LDB;
   constexpr bool IS_BF16 = sizeof(T) == 2;
   constexpr bool FWD = MODE != MODE_BWDX;
 
-  __shared__ __attribute__((aligned(16))) T sA[kTileRows * LDA];
-  __shared__ __attribute__((aligned(16))) T sB[B_ELEMS];
+  __shared__ __attribute__((aligned(16))) T sA[2 * A_ELEMS];   // two stages
+  __shared__ __attribute__((aligned(16))) T sB[2 * B_ELEMS];
   __shared__ __attribute__((aligned(16))) float sCol[4][kTileCols];
   __shared__ float sRed[2][kTileRows];
   __shared__ int sCnt[4];
@@ -64,12 +73,13 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
   const int wr = wave >> 1, wc = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  const int row_tile = blockIdx.x / p.n_col_blocks;
-  const int cb = blockIdx.x % p.n_col_blocks;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int row_tile = lid / p.n_col_blocks;
+  const int cb = lid % p.n_col_blocks;
   find_row_tile(p.offsets, p.E, row_tile, sInfo, sWave);
   const int e = sInfo[0];
   if (e < 0) {
-    if (MODE == MODE_BWDX && tid == 0 && p.notclip_count) p.notclip_count[blockIdx.x] = 0;
+    if (MODE == MODE_BWDX && tid == 0 && p.notclip_count) p.notclip_count[lid] = 0;
     return;
   }
   const int row0 = sInfo[1], row_end = sInfo[2];
@@ -83,10 +93,12 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
   const bool has_ir = FWD && p.ir != nullptr;
   const bool has_amax = FWD && p.abs_max != nullptr;
   const bool quant = FWD && p.inp_res > 0.f;
+  const bool dac = has_ir || has_amax || quant;
   const bool codes_mode = IS_BF16 && quant;   // feed integer codes, scale the accumulator
   const bool adc_clip = FWD && p.out_bound > 0.f;
   const bool adc_quant = adc_clip && p.out_half_states > 0.f;
   const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
+  const float inv_res = quant ? 1.0f / p.inp_res : 0.f;
 
   // ---- per-column constants of the forward epilogue --------------------------------------
   if (FWD && tid < kTileCols) {
@@ -105,14 +117,16 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
   const int a_chunk = tid & 7;
   const T* a_row[4];
   bool a_ok[4];
-  float a_amax[4];
+  float a_amax[4], a_amax_inv[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int r = row0 + (tid >> 3) + 32 * i;
     a_ok[i] = r < row_end;
-    const int idx = a_ok[i] ? p.a_index[r] : 0;
+    // rows past the tile read the tile's first row: safe to load, never stored
+    const int idx = p.a_index[a_ok[i] ? r : row0];
     a_row[i] = A + (int64_t)idx * p.lda;
     a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[idx] : 1.f;
+    a_amax_inv[i] = 1.0f / a_amax[i];
   }
   // RC weights: thread -> contraction rows tid/CPR + RPP*i, chunk tid%CPR of the 128 columns.
   constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
@@ -132,11 +146,12 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
   for (int t = 0; t < p.n_kd_tiles; t++) {
     const int klo = p.kd_bounds[t], khi = p.kd_bounds[t + 1];
     const int nsteps = (khi - klo + BK - 1) / BK;
-    float a_ir[4];
+    float a_ir[4], a_ir_inv[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int r = row0 + (tid >> 3) + 32 * i;
       a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
+      a_ir_inv[i] = 1.0f / a_ir[i];
     }
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -145,15 +160,29 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
 
-    Chunk<T> ra[4], rb[4];
-    auto load_step = [&](int s) {
+    Raw ra[4], rb[4];
+    // Interior tiles (every chunk complete and 16-byte aligned) take unconditional vector loads.
+    const bool fast = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
+    const T* wp[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      wp[i] = W_KC ? W + (int64_t)(c0 + (tid >> 3) + 32 * i) * p.w_snd + klo + a_chunk * CH
+                   : W + (int64_t)(klo + tid / CPR + RPP * i) * p.w_skd + c0 + (tid % CPR) * CH;
+    const int64_t w_step = W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd;
+    auto load_fast = [&](int s) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) ra[i] = *reinterpret_cast<const Raw*>(a_row[i] + klo + s * BK + a_chunk * CH);
+#pragma unroll
+      for (int i = 0; i < 4; i++) rb[i] = *reinterpret_cast<const Raw*>(wp[i] + s * w_step);
+    };
+    auto load_step = [&](int s) {          // global -> registers, any shape
       const int k0 = klo + s * BK;
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int kpos = k0 + a_chunk * CH;
         int nv = a_ok[i] ? khi - kpos : 0;
         nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-        ra[i] = chunk_load<T>(a_row[i] + kpos, nv, p.a_vec != 0);
+        ra[i] = raw_load<T>(a_row[i] + kpos, nv, p.a_vec != 0);
       }
       if (W_KC) {
 #pragma unroll
@@ -162,7 +191,7 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
           const int kpos = k0 + a_chunk * CH;
           int nv = col < c1 ? khi - kpos : 0;
           nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-          rb[i] = chunk_load<T>(W + (int64_t)col * p.w_snd + kpos, nv, p.w_vec != 0);
+          rb[i] = raw_load<T>(W + (int64_t)col * p.w_snd + kpos, nv, p.w_vec != 0);
         }
       } else {
 #pragma unroll
@@ -171,60 +200,72 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
           const int col = c0 + (tid % CPR) * CH;
           int nv = kd < khi ? c1 - col : 0;
           nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-          rb[i] = chunk_load<T>(W + (int64_t)kd * p.w_skd + col, nv, p.w_vec != 0);
+          rb[i] = raw_load<T>(W + (int64_t)kd * p.w_skd + col, nv, p.w_vec != 0);
         }
       }
     };
-
-    load_step(0);
-    for (int s = 0; s < nsteps; s++) {
-      // ---- prologue on the gathered rows, then registers -> LDS ------------------------------
+    auto store_step = [&](int buf) {       // registers -> LDS stage buf, DAC stage on the way
+      T* __restrict__ dA = sA + buf * A_ELEMS;
+      T* __restrict__ dB = sB + buf * B_ELEMS;
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        if (FWD && (has_ir || has_amax || quant)) {
+        Raw a = ra[i];
+        if (FWD && dac) {
+          float v[CH];
+          raw_unpack<T>(a, v);
           bool out_of_range = false;
 #pragma unroll
           for (int j = 0; j < CH; j++) {
-            float v = ra[i].v[j];
+            float x = v[j];
             if (has_ir) {
               const float r = a_ir[i];
-              v = v > r ? r : v;
-              v = v < -r ? -r : v;
-              v = v / r;
+              x = x > r ? r : x;
+              x = x < -r ? -r : x;
+              x = div_by(x, r, a_ir_inv[i]);
             }
-            if (has_amax) v = v / a_amax[i];
+            if (has_amax) x = div_by(x, a_amax[i], a_amax_inv[i]);
             if (quant) {
-              out_of_range |= !(fabsf(v) <= 1.0f);
-              v = rintf(v / p.inp_res);
-              if (!IS_BF16) v = v * p.inp_res;
+              out_of_range |= !(fabsf(x) <= 1.0f);
+              x = rintf(div_by(x, p.inp_res, inv_res));
+              if (!IS_BF16) x = x * p.inp_res;
             }
-            ra[i].v[j] = v;
+            v[j] = x;
           }
           if (quant && out_of_range && a_ok[i] && p.range_flag != nullptr) atomicOr(p.range_flag, 1);
+          if constexpr (IS_BF16) a = codes_mode ? raw_pack_exact_bf16(v) : raw_pack<T>(v);
+          else a = raw_pack<T>(v);
         }
-        chunk_store_lds<T>(&sA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH], ra[i]);
-        if (W_KC) chunk_store_lds<T>(&sB[((tid >> 3) + 32 * i) * LDB + a_chunk * CH], rb[i]);
-        else chunk_store_lds<T>(&sB[(tid / CPR + RPP * i) * LDB + (tid % CPR) * CH], rb[i]);
+        *reinterpret_cast<Raw*>(&dA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH]) = a;
+        if (W_KC) *reinterpret_cast<Raw*>(&dB[((tid >> 3) + 32 * i) * LDB + a_chunk * CH]) = rb[i];
+        else *reinterpret_cast<Raw*>(&dB[(tid / CPR + RPP * i) * LDB + (tid % CPR) * CH]) = rb[i];
       }
-      __syncthreads();
-      if (s + 1 < nsteps) load_step(s + 1);
+    };
 
-      // ---- matrix instructions -----------------------------------------------------------------
+    if (fast) load_fast(0); else load_step(0);
+    store_step(0);
+    __syncthreads();
+    for (int s = 0; s < nsteps; s++) {
+      const int cur = s & 1;
+      if (s + 1 < nsteps) {                   // in flight while this stage is multiplied
+        if (fast) load_fast(s + 1); else load_step(s + 1);
+      }
+      const T* __restrict__ cA = sA + cur * A_ELEMS;
+      const T* __restrict__ cB = sB + cur * B_ELEMS;
 #pragma unroll
       for (int kk = 0; kk < BK; kk += MMAK) {
         if constexpr (IS_BF16) {
           u32x4 xf[2], wf[2];
 #pragma unroll
           for (int ti = 0; ti < 2; ti++)
-            xf[ti] = *reinterpret_cast<const u32x4*>(&sA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
+            xf[ti] = *reinterpret_cast<const u32x4*>(&cA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
 #pragma unroll
           for (int fi = 0; fi < 2; fi++) {
             if (W_KC) {
-              wf[fi] = *reinterpret_cast<const u32x4*>(&sB[(wc * 64 + fi * 32 + l32) * LDB + kk + 8 * lh]);
+              wf[fi] = *reinterpret_cast<const u32x4*>(&cB[(wc * 64 + fi * 32 + l32) * LDB + kk + 8 * lh]);
             } else {
               const int R = lane & 15, g = (lane >> 4) & 1;
               const uint16_t* base = reinterpret_cast<const uint16_t*>(
-                  &sB[(kk + 8 * lh + (R >> 2)) * LDB + wc * 64 + fi * 32 + 16 * g + 4 * (R & 3)]);
+                  &cB[(kk + 8 * lh + (R >> 2)) * LDB + wc * 64 + fi * 32 + 16 * g + 4 * (R & 3)]);
               u32x2 lo = lds_read_tr16_b64(base);
               u32x2 hi = lds_read_tr16_b64(base + 4 * LDB);
               wf[fi] = u32x4{lo[0], lo[1], hi[0], hi[1]};
@@ -237,17 +278,18 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
         } else {
           float xf[2], wf[2];
 #pragma unroll
-          for (int ti = 0; ti < 2; ti++) xf[ti] = sA[(wr * 64 + ti * 32 + l32) * LDA + kk + lh];
+          for (int ti = 0; ti < 2; ti++) xf[ti] = cA[(wr * 64 + ti * 32 + l32) * LDA + kk + lh];
 #pragma unroll
           for (int fi = 0; fi < 2; fi++)
-            wf[fi] = W_KC ? sB[(wc * 64 + fi * 32 + l32) * LDB + kk + lh]
-                          : sB[(kk + lh) * LDB + wc * 64 + fi * 32 + l32];
+            wf[fi] = W_KC ? cB[(wc * 64 + fi * 32 + l32) * LDB + kk + lh]
+                          : cB[(kk + lh) * LDB + wc * 64 + fi * 32 + l32];
 #pragma unroll
           for (int fi = 0; fi < 2; fi++)
 #pragma unroll
             for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x2_f32(wf[fi], xf[ti], acc[fi][ti]);
         }
       }
+      if (s + 1 < nsteps) store_step(cur ^ 1);
       __syncthreads();
     }
 
@@ -392,7 +434,7 @@ __global__ __launch_bounds__(kThreads) void gemm_rows_kernel(const RowsParams p)
       __syncthreads();
       if (tid < kTileRows && row0 + tid < row_end)
         p.irg_partial[(int64_t)cb * p.M + row0 + tid] = sRed[0][tid] + sRed[1][tid];
-      if (tid == 0) p.notclip_count[blockIdx.x] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
+      if (tid == 0) p.notclip_count[lid] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
     }
   }
 }

@@ -7,6 +7,7 @@
 // gradient fragment is the A operand, so a lane holds one kk and runs of 4 consecutive n.
 #pragma once
 #include "common.h"
+#include "gemm_rows.h"
 
 namespace amoe {
 
@@ -22,23 +23,24 @@ struct WgradParams {
 };
 
 template <typename T>
-__global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams p) {
+__global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradParams p) {
   using EL = Elem<T>;
   constexpr int CH = EL::kChunk, MMAK = EL::kMmaK;
   constexpr int BT = EL::kBK;                     // tokens per step
   constexpr int LD = kTileCols + EL::kPadRC;
+  constexpr int STAGE = BT * LD;
   constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
   constexpr bool IS_BF16 = sizeof(T) == 2;
   static_assert(BT == 4 * RPP, "staging expects 4 passes");
 
-  __shared__ __attribute__((aligned(16))) T sX[BT * LD];
-  __shared__ __attribute__((aligned(16))) T sG[BT * LD];
+  __shared__ __attribute__((aligned(16))) T sX[2 * STAGE];   // two stages
+  __shared__ __attribute__((aligned(16))) T sG[2 * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave >> 1, wk = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  int b = blockIdx.x;
+  int b = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int nb = b % p.n_n_blocks; b /= p.n_n_blocks;
   const int kb = b % p.n_k_blocks;
   const int e = b / p.n_k_blocks;
@@ -52,6 +54,7 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
   const T* __restrict__ GS = static_cast<const T*>(p.g_scale);
   const bool has_ir = p.ir != nullptr;
   const int chunk = tid % CPR;
+  const float ir_expert = (has_ir && p.ir_by_expert) ? p.ir[(int64_t)e * p.n_tiles + kcol.tile] : 1.f;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -61,49 +64,93 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][c][i] = 0.f;
 
-  Chunk<T> rx[4], rg[4];
-  auto load_step = [&](int i0) {
+  // rows of the step after the one being loaded: indices are fetched one step ahead of the data
+  int nx_xi[4], nx_gi[4];
+  float nx_ir[4];
+  bool nx_ok[4];
+  auto load_index = [&](int i0) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int r = i0 + tid / CPR + RPP * i;
-      const bool ok = r < seg1;
-      const int xi = ok ? p.in_index[r] : 0;
-      const int gi = ok ? (p.g_index ? p.g_index[r] : xi) : 0;
+      nx_ok[i] = r < seg1;
+      nx_xi[i] = nx_ok[i] ? p.in_index[r] : 0;
+      nx_gi[i] = nx_ok[i] ? (p.g_index ? p.g_index[r] : nx_xi[i]) : 0;
+      nx_ir[i] = (has_ir && !p.ir_by_expert && nx_ok[i]) ? p.ir[(int64_t)r * p.n_tiles + kcol.tile] : ir_expert;
+    }
+  };
+  Raw rx[4], rg[4];
+  float st_ir[4], st_gs[4];
+  auto load_step = [&]() {                   // global -> registers, rows from nx_*
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
       const int kk = kc0 + chunk * CH;
-      int nvx = ok ? kc1 - kk : 0;
+      int nvx = nx_ok[i] ? kc1 - kk : 0;
       nvx = nvx < 0 ? 0 : (nvx > CH ? CH : nvx);
-      rx[i] = chunk_load<T>(X + (int64_t)xi * p.ldx + kk, nvx, p.x_vec != 0);
-      if (has_ir && ok) {
-        const float rng = p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.n_tiles + kcol.tile];
+      rx[i] = raw_load<T>(X + (int64_t)nx_xi[i] * p.ldx + kk, nvx, p.x_vec != 0);
+      const int n = n0 + chunk * CH;
+      int nvg = nx_ok[i] ? n1 - n : 0;
+      nvg = nvg < 0 ? 0 : (nvg > CH ? CH : nvg);
+      rg[i] = raw_load<T>(G + (int64_t)nx_gi[i] * p.ldg + n, nvg, p.g_vec != 0);
+      st_ir[i] = nx_ir[i];
+      st_gs[i] = (GS != nullptr && nx_ok[i]) ? Elem<T>::load(GS + nx_xi[i]) : 1.f;
+    }
+  };
+  // Interior steps (all BT tokens exist, full 128-column tiles, aligned rows): unconditional loads.
+  const bool tile_fast = p.x_vec != 0 && p.g_vec != 0 && (kc1 - kc0) == kTileCols && (n1 - n0) == kTileCols;
+  auto load_fast = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      rx[i] = *reinterpret_cast<const Raw*>(X + (int64_t)nx_xi[i] * p.ldx + kc0 + chunk * CH);
+      rg[i] = *reinterpret_cast<const Raw*>(G + (int64_t)nx_gi[i] * p.ldg + n0 + chunk * CH);
+      st_ir[i] = nx_ir[i];
+      st_gs[i] = GS != nullptr ? Elem<T>::load(GS + nx_xi[i]) : 1.f;
+    }
+  };
+  auto store_step = [&](int buf) {           // registers -> LDS, clip / gate scaling on the way
+    T* __restrict__ dX = sX + buf * STAGE;
+    T* __restrict__ dG = sG + buf * STAGE;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      Raw x = rx[i], g = rg[i];
+      if (has_ir) {
+        float v[CH];
+        raw_unpack<T>(x, v);
+        const float rng = st_ir[i];
 #pragma unroll
         for (int j = 0; j < CH; j++) {
-          float v = rx[i].v[j];
-          v = v > rng ? rng : v;
-          v = v < -rng ? -rng : v;
-          rx[i].v[j] = v;
+          v[j] = v[j] > rng ? rng : v[j];
+          v[j] = v[j] < -rng ? -rng : v[j];
         }
+        x = raw_pack<T>(v);
       }
-      const int n = n0 + chunk * CH;
-      int nvg = ok ? n1 - n : 0;
-      nvg = nvg < 0 ? 0 : (nvg > CH ? CH : nvg);
-      rg[i] = chunk_load<T>(G + (int64_t)gi * p.ldg + n, nvg, p.g_vec != 0);
-      if (GS != nullptr && ok) {
-        const float sc = Elem<T>::load(GS + xi);
+      if (GS != nullptr) {
+        float v[CH];
+        raw_unpack<T>(g, v);
 #pragma unroll
-        for (int j = 0; j < CH; j++) rg[i].v[j] *= sc;
+        for (int j = 0; j < CH; j++) v[j] *= st_gs[i];
+        g = raw_pack<T>(v);
       }
+      *reinterpret_cast<Raw*>(&dX[(tid / CPR + RPP * i) * LD + chunk * CH]) = x;
+      *reinterpret_cast<Raw*>(&dG[(tid / CPR + RPP * i) * LD + chunk * CH]) = g;
     }
   };
 
-  if (seg0 < seg1) load_step(seg0);
+  if (seg0 < seg1) {
+    load_index(seg0);
+    if (tile_fast && seg0 + BT <= seg1) load_fast(); else load_step();
+    load_index(seg0 + BT);
+    store_step(0);
+  }
+  __syncthreads();
+  int cur = 0;
   for (int i0 = seg0; i0 < seg1; i0 += BT) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      chunk_store_lds<T>(&sX[(tid / CPR + RPP * i) * LD + chunk * CH], rx[i]);
-      chunk_store_lds<T>(&sG[(tid / CPR + RPP * i) * LD + chunk * CH], rg[i]);
+    const bool more = i0 + BT < seg1;
+    if (more) {
+      if (tile_fast && i0 + 2 * BT <= seg1) load_fast(); else load_step();
+      load_index(i0 + 2 * BT);
     }
-    __syncthreads();
-    if (i0 + BT < seg1) load_step(i0 + BT);
+    const T* __restrict__ cX = sX + cur * STAGE;
+    const T* __restrict__ cG = sG + cur * STAGE;
 #pragma unroll
     for (int kk = 0; kk < BT; kk += MMAK) {
       if constexpr (IS_BF16) {
@@ -112,8 +159,8 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
         u32x4 gf[2], xf[2];
 #pragma unroll
         for (int f = 0; f < 2; f++) {
-          const uint16_t* bg = reinterpret_cast<const uint16_t*>(&sG[roff + wn * 64 + f * 32]);
-          const uint16_t* bx = reinterpret_cast<const uint16_t*>(&sX[roff + wk * 64 + f * 32]);
+          const uint16_t* bg = reinterpret_cast<const uint16_t*>(&cG[roff + wn * 64 + f * 32]);
+          const uint16_t* bx = reinterpret_cast<const uint16_t*>(&cX[roff + wk * 64 + f * 32]);
           u32x2 glo = lds_read_tr16_b64(bg), ghi = lds_read_tr16_b64(bg + 4 * LD);
           u32x2 xlo = lds_read_tr16_b64(bx), xhi = lds_read_tr16_b64(bx + 4 * LD);
           gf[f] = u32x4{glo[0], glo[1], ghi[0], ghi[1]};
@@ -127,8 +174,8 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
         float gf[2], xf[2];
 #pragma unroll
         for (int f = 0; f < 2; f++) {
-          gf[f] = sG[(kk + lh) * LD + wn * 64 + f * 32 + l32];
-          xf[f] = sX[(kk + lh) * LD + wk * 64 + f * 32 + l32];
+          gf[f] = cG[(kk + lh) * LD + wn * 64 + f * 32 + l32];
+          xf[f] = cX[(kk + lh) * LD + wk * 64 + f * 32 + l32];
         }
 #pragma unroll
         for (int fn = 0; fn < 2; fn++)
@@ -136,7 +183,9 @@ __global__ __launch_bounds__(kThreads) void gemm_wgrad_kernel(const WgradParams 
           for (int fk = 0; fk < 2; fk++) acc[fn][fk] = mfma_32x32x2_f32(gf[fn], xf[fk], acc[fn][fk]);
       }
     }
+    if (more) store_step(cur ^ 1);
     __syncthreads();
+    cur ^= 1;
   }
 
   T* __restrict__ GW = static_cast<T*>(p.grad_w) + (int64_t)e * p.K * p.N;

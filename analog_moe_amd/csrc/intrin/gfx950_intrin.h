@@ -55,6 +55,14 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Two fp32 -> packed bf16 (round to nearest even), one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 // sin / cos of 2*pi*x (x in revolutions), natural log, sqrt: single hardware instructions.
 __device__ __forceinline__ float fast_sin_rev(float x) { return __builtin_amdgcn_sinf(x); }
 __device__ __forceinline__ float fast_cos_rev(float x) { return __builtin_amdgcn_cosf(x); }

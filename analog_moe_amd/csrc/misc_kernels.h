@@ -70,20 +70,32 @@ __global__ __launch_bounds__(kThreads) void weight_col_abs_max_kernel(const T* _
   for (int k = 0; k < K; k++) m = fmaxf(m, fabsf(Elem<T>::load(base + (long long)k * N)));
   out[(long long)e * N + c] = m;
 }
-// cols == 1: wmax[e] = max |w[e]|, one workgroup per expert.
+// cols == 1: wmax[e] = max |w[e]|.  grid (chunks, E): every workgroup reduces one slice and
+// merges with an atomic max on the bit pattern (non-negative floats order like integers), so the
+// output must be zero-filled first (fill_zero_kernel).
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restrict__ p, int n) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
 template <typename T>
 __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __restrict__ w, long long per_expert,
                                                                    float* __restrict__ out) {
   __shared__ float red[4];
   const int tid = threadIdx.x, lane = tid & 63;
-  const T* base = w + (long long)blockIdx.x * per_expert;
+  const T* base = w + (long long)blockIdx.y * per_expert;
+  const long long span = (per_expert + gridDim.x - 1) / gridDim.x;
+  const long long lo = (long long)blockIdx.x * span;
+  const long long hi = lo + span < per_expert ? lo + span : per_expert;
   float m = 0.f;
-  for (long long i = tid; i < per_expert; i += kThreads) m = fmaxf(m, fabsf(Elem<T>::load(base + i)));
+  for (long long i = lo + tid; i < hi; i += kThreads) m = fmaxf(m, fabsf(Elem<T>::load(base + i)));
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, wave_shfl_xor(m, d));
   if (lane == 0) red[tid >> 6] = m;
   __syncthreads();
-  if (tid == 0) out[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  if (tid == 0) {
+    const float r = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    atomicMax(reinterpret_cast<uint32_t*>(out) + blockIdx.y, as_u32(r));
+  }
 }
 
 // out[e, t] = sum_{i in [offsets[e], offsets[e+1])} v[i, t], one workgroup per (expert, tile).

@@ -109,6 +109,15 @@ inline u32x2 lds_read_tr16_b64(const uint16_t* p) {
   return out;
 }
 
+inline uint32_t emu_f32_to_bf16(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+inline uint32_t pack_bf16x2(float lo, float hi) { return emu_f32_to_bf16(lo) | (emu_f32_to_bf16(hi) << 16); }
+
 inline float fast_sin_rev(float x) { return sinf(6.283185307179586f * x); }
 inline float fast_cos_rev(float x) { return cosf(6.283185307179586f * x); }
 inline float fast_log(float x) { return logf(x); }
