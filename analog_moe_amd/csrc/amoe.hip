@@ -30,6 +30,29 @@ inline bool bounds_multiple_of(int n_tiles, const int32_t* b, int m) {
 inline size_t esize(int dtype) { return dtype == AMOE_F32 ? 4 : 2; }
 inline int max_row_tiles(int64_t M, int E) { return (int)(M / kTileRows) + E; }
 
+// Compute units of the current device (read once; the value cannot change while the process lives).
+inline int num_compute_units() {
+  static const int n = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) return 256;
+    return cu;
+  }();
+  return n;
+}
+
+// Persistent grid of the row-gather GEMM: two workgroups per compute unit, more if a workgroup
+// would otherwise own more row tiles than its descriptor table holds, never more than work items.
+inline int persistent_grid(int row_tiles, int col_blocks) {
+  const long long work = (long long)row_tiles * col_blocks;
+  long long g = 2LL * num_compute_units();
+  const long long cap = (long long)(kMaxDesc - 2) * col_blocks;
+  const long long need = (work + cap - 1) / cap;
+  if (need > g) g = need;
+  if (g > work) g = work;
+  return g < 1 ? 1 : (int)g;
+}
+
 template <typename T, bool W_KC>
 int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
   if (mode == MODE_FWD) {
@@ -160,7 +183,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
                   : (a->w_stride_k % CH == 0));
   p.out_vec = aligned(a->out, 16) && (a->ldo % 4 == 0);
   p.noise_vec = a->noise && aligned(a->noise, 16) && (a->ldnoise % 4 == 0) && (a->noise_tile_stride % 4 == 0);
-  const int grid = max_row_tiles(a->M, a->E) * p.n_col_blocks;
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (a->dtype == AMOE_F32)
@@ -244,8 +267,7 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles);
   p.ir = a->ir; p.ir_cols = a->n_tiles; p.ir_by_expert = a->ir_by_expert; p.inp_res = -1.f;
   p.xf = a->x; p.ldxf = a->ldx; p.xf_index = a->xf_index; p.gate = a->gate; p.relu_mask = a->relu_mask;
-  const int row_tiles = max_row_tiles(a->M, a->E);
-  const int grid = row_tiles * p.n_col_blocks;
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (use_ir) {
     const size_t need = (size_t)p.n_col_blocks * a->M * sizeof(float) + (size_t)grid * sizeof(int32_t);
     if (a->workspace_bytes < need) return AMOE_EWORKSPACE;

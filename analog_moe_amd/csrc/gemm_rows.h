@@ -50,6 +50,11 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int grid) {
   return xcd * q + (xcd < r ? xcd : r) + idx;
 }
 
+constexpr int kMaxDesc = 64;   // row tiles one workgroup can own (the host sizes the grid for it)
+
+// Persistent workgroups: the list of work items (row tile, column block), column block fastest,
+// is cut into gridDim.x contiguous ranges; a workgroup walks its range, keeping the row tile's
+// gather pointers while only the column block changes.
 template <typename T, bool W_KC, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams p) {
   using EL = Elem<T>;
@@ -58,384 +63,508 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   constexpr int LDB = W_KC ? (BK + EL::kPadKC) : (kTileCols + EL::kPadRC);
   constexpr int A_ELEMS = kTileRows * LDA;
   constexpr int B_ELEMS = W_KC ? kTileCols * LDB : BK * LDB;
+  constexpr int STAGE = A_ELEMS + B_ELEMS;
   constexpr bool IS_BF16 = sizeof(T) == 2;
   constexpr bool FWD = MODE != MODE_BWDX;
+  // output staging in LDS: rows of 128 columns + 16 bytes, as many rows per pass as one stage holds
+  constexpr int LDO = kTileCols + 16 / (int)sizeof(T);
+  constexpr int OUT_PASSES = IS_BF16 ? 1 : 2;
+  constexpr int OUT_ROWS = kTileRows / OUT_PASSES;
+  static_assert(OUT_ROWS * LDO <= 2 * STAGE, "output staging must fit the stage buffers");
 
-  __shared__ __attribute__((aligned(16))) T sA[2 * A_ELEMS];   // two stages
-  __shared__ __attribute__((aligned(16))) T sB[2 * B_ELEMS];
+  __shared__ __attribute__((aligned(16))) T sStage[2 * STAGE];
   __shared__ __attribute__((aligned(16))) float sCol[4][kTileCols];
   __shared__ float sRed[2][kTileRows];
+  __shared__ int sOrow[kTileRows];
+  __shared__ int sDesc[kMaxDesc][4];
   __shared__ int sCnt[4];
-  __shared__ int sInfo[8];
   __shared__ int sWave[4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave >> 1, wc = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
+  const int ncb = p.n_col_blocks;
 
-  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int row_tile = lid / p.n_col_blocks;
-  const int cb = lid % p.n_col_blocks;
-  find_row_tile(p.offsets, p.E, row_tile, sInfo, sWave);
-  const int e = sInfo[0];
-  if (e < 0) {
-    if (MODE == MODE_BWDX && tid == 0 && p.notclip_count) p.notclip_count[lid] = 0;
-    return;
+  // ---- this workgroup's range of work items ----------------------------------------------------
+  // tiles per expert -> exclusive prefix (thread tid owns experts [tid*per, (tid+1)*per))
+  const int per = (p.E + kThreads - 1) / kThreads;
+  const int e_first = tid * per;
+  int mine = 0;
+  for (int j = 0; j < per; j++) {
+    const int e = e_first + j;
+    if (e < p.E) mine += (p.offsets[e + 1] - p.offsets[e] + kTileRows - 1) / kTileRows;
   }
-  const int row0 = sInfo[1], row_end = sInfo[2];
-  const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb);
-  const int c0 = colb.c0, c1 = colb.c1;
+  int incl = mine;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = wave_shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == 63) sWave[wave] = incl;
+  __syncthreads();
+  int tiles_before = incl - mine;
+  for (int w = 0; w < wave; w++) tiles_before += sWave[w];
+  const int total_rt = sWave[0] + sWave[1] + sWave[2] + sWave[3];
+  const int total_work = total_rt * ncb;
+  const int lb = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int share = total_work / (int)gridDim.x, extra = total_work % (int)gridDim.x;
+  const int w0 = lb * share + (lb < extra ? lb : extra);
+  const int w1 = w0 + share + (lb < extra ? 1 : 0);
+  int cnt = 0;                                       // un-clipped inputs seen by this lane (MODE_BWDX)
+  if (w0 < w1) {
+    const int rt_first = w0 / ncb, rt_last = (w1 - 1) / ncb;
+    // descriptors (expert, first sorted position, end position) of the row tiles of the range
+    int t = tiles_before;
+    for (int j = 0; j < per; j++) {
+      const int e = e_first + j;
+      if (e < p.E) {
+        const int lo = p.offsets[e], hi = p.offsets[e + 1];
+        const int nt = (hi - lo + kTileRows - 1) / kTileRows;
+        int a = rt_first > t ? rt_first : t;
+        const int b = rt_last < t + nt - 1 ? rt_last : t + nt - 1;
+        for (; a <= b; a++) {
+          const int slot = a - rt_first;
+          if (slot < kMaxDesc) {
+            const int r0 = lo + (a - t) * kTileRows;
+            sDesc[slot][0] = e;
+            sDesc[slot][1] = r0;
+            sDesc[slot][2] = r0 + kTileRows < hi ? r0 + kTileRows : hi;
+          }
+        }
+        t += nt;
+      }
+    }
+  }
+  __syncthreads();
 
   const T* __restrict__ A = static_cast<const T*>(p.a);
-  const T* __restrict__ W = static_cast<const T*>(p.w) + (int64_t)e * p.w_se;
   T* __restrict__ OUT = static_cast<T*>(p.out);
-
   const bool has_ir = FWD && p.ir != nullptr;
   const bool has_amax = FWD && p.abs_max != nullptr;
   const bool quant = FWD && p.inp_res > 0.f;
   const bool dac = has_ir || has_amax || quant;
+  const bool dac_ir_quant = has_ir && quant && !has_amax;   // the common analog case: tight code
   const bool codes_mode = IS_BF16 && quant;   // feed integer codes, scale the accumulator
   const bool adc_clip = FWD && p.out_bound > 0.f;
   const bool adc_quant = adc_clip && p.out_half_states > 0.f;
   const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
   const float inv_res = quant ? 1.0f / p.inp_res : 0.f;
+  const bool use_ir_bw = !FWD && p.ir != nullptr;
 
-  // ---- per-column constants of the forward epilogue --------------------------------------
-  if (FWD && tid < kTileCols) {
-    const int col = c0 + tid;
-    float wm = 1.f;
-    if (p.wmax != nullptr && col < c1) wm = p.wmax[(int64_t)e * p.wmax_cols + (p.wmax_cols > 1 ? col : 0)];
-    const float bound = p.out_bound * wm;
-    sCol[0][tid] = p.noise_std * wm;
-    sCol[1][tid] = bound;
-    sCol[2][tid] = adc_quant ? p.out_half_states / bound : 0.f;
-    sCol[3][tid] = adc_quant ? bound / p.out_half_states : 0.f;
-  }
-
-  // ---- staging assignments ------------------------------------------------------------------
-  // A (and KC weights): thread -> rows tid/8 + 32*i (i < 4), 16-byte chunk tid%8 of the step.
   const int a_chunk = tid & 7;
+  constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
+  static_assert(BK == 4 * RPP, "RC staging expects 4 passes");
+
+  // state of the current row tile
+  int e = 0, row0 = 0, row_end = 0, cur_rt = -1;
   const T* a_row[4];
   bool a_ok[4];
   float a_amax[4], a_amax_inv[4];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int r = row0 + (tid >> 3) + 32 * i;
-    a_ok[i] = r < row_end;
-    // rows past the tile read the tile's first row: safe to load, never stored
-    const int idx = p.a_index[a_ok[i] ? r : row0];
-    a_row[i] = A + (int64_t)idx * p.lda;
-    a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[idx] : 1.f;
-    a_amax_inv[i] = 1.0f / a_amax[i];
-  }
-  // RC weights: thread -> contraction rows tid/CPR + RPP*i, chunk tid%CPR of the 128 columns.
-  constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
-  static_assert(BK == 4 * RPP, "RC staging expects 4 passes");
+  for (int i = 0; i < 4; i++) { a_row[i] = A; a_ok[i] = false; a_amax[i] = a_amax_inv[i] = 1.f; }
 
-  f32x16 acc[2][2];
-  f32x16 total[2][2];
-  if (MODE == MODE_FWD_SPLIT) {
+  for (int w = w0; w < w1; w++) {
+    const int rt = w / ncb, cb = w - rt * ncb;
+    if (rt != cur_rt) {                     // new row tile: gather pointers, scatter rows
+      cur_rt = rt;
+      const int slot = rt - w0 / ncb;
+      e = sDesc[slot][0]; row0 = sDesc[slot][1]; row_end = sDesc[slot][2];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
-#pragma unroll
-      for (int b = 0; b < 2; b++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) total[a][b][i] = 0.f;
-  }
-
-  for (int t = 0; t < p.n_kd_tiles; t++) {
-    const int klo = p.kd_bounds[t], khi = p.kd_bounds[t + 1];
-    const int nsteps = (khi - klo + BK - 1) / BK;
-    float a_ir[4], a_ir_inv[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int r = row0 + (tid >> 3) + 32 * i;
-      a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
-      a_ir_inv[i] = 1.0f / a_ir[i];
+      for (int i = 0; i < 4; i++) {
+        const int r = row0 + (tid >> 3) + 32 * i;
+        a_ok[i] = r < row_end;
+        // rows past the tile read the tile's first row: safe to load, never stored
+        const int idx = p.a_index[a_ok[i] ? r : row0];
+        a_row[i] = A + (int64_t)idx * p.lda;
+        a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[idx] : 1.f;
+        a_amax_inv[i] = 1.0f / a_amax[i];
+      }
+      if (tid < kTileRows) {
+        const int r = row0 + tid;
+        sOrow[tid] = r < row_end ? (p.out_index ? p.out_index[r] : p.a_index[r]) : -1;
+      }
     }
-#pragma unroll
-    for (int a = 0; a < 2; a++)
-#pragma unroll
-      for (int b = 0; b < 2; b++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+    const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb);
+    const int c0 = colb.c0, c1 = colb.c1;
+    const T* __restrict__ W = static_cast<const T*>(p.w) + (int64_t)e * p.w_se;
 
-    Raw ra[4], rb[4];
-    // Interior tiles (every chunk complete and 16-byte aligned) take unconditional vector loads.
-    const bool fast = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
-    const T* wp[4];
+    // per-column constants of the forward epilogue (last read before the barrier that ended the
+    // previous item)
+    if (FWD && tid < kTileCols) {
+      const int col = c0 + tid;
+      float wm = 1.f;
+      if (p.wmax != nullptr && col < c1) wm = p.wmax[(int64_t)e * p.wmax_cols + (p.wmax_cols > 1 ? col : 0)];
+      const float bound = p.out_bound * wm;
+      sCol[0][tid] = p.noise_std * wm;
+      sCol[1][tid] = bound;
+      sCol[2][tid] = adc_quant ? p.out_half_states / bound : 0.f;
+      sCol[3][tid] = adc_quant ? bound / p.out_half_states : 0.f;
+    }
+
+    f32x16 acc[2][2];
+    f32x16 total[2][2];
+    if (MODE == MODE_FWD_SPLIT) {
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      wp[i] = W_KC ? W + (int64_t)(c0 + (tid >> 3) + 32 * i) * p.w_snd + klo + a_chunk * CH
-                   : W + (int64_t)(klo + tid / CPR + RPP * i) * p.w_skd + c0 + (tid % CPR) * CH;
-    const int64_t w_step = W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd;
-    auto load_fast = [&](int s) {
+      for (int a = 0; a < 2; a++)
 #pragma unroll
-      for (int i = 0; i < 4; i++) ra[i] = *reinterpret_cast<const Raw*>(a_row[i] + klo + s * BK + a_chunk * CH);
+        for (int b = 0; b < 2; b++)
 #pragma unroll
-      for (int i = 0; i < 4; i++) rb[i] = *reinterpret_cast<const Raw*>(wp[i] + s * w_step);
-    };
-    auto load_step = [&](int s) {          // global -> registers, any shape
-      const int k0 = klo + s * BK;
+          for (int i = 0; i < 16; i++) total[a][b][i] = 0.f;
+    }
+
+    for (int t = 0; t < p.n_kd_tiles; t++) {
+      const int klo = p.kd_bounds[t], khi = p.kd_bounds[t + 1];
+      const int nsteps = (khi - klo + BK - 1) / BK;
+      float a_ir[4], a_ir_inv[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        const int kpos = k0 + a_chunk * CH;
-        int nv = a_ok[i] ? khi - kpos : 0;
-        nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-        ra[i] = raw_load<T>(a_row[i] + kpos, nv, p.a_vec != 0);
+        const int r = row0 + (tid >> 3) + 32 * i;
+        a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
+        a_ir_inv[i] = 1.0f / a_ir[i];
       }
-      if (W_KC) {
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+
+      Raw ra[4], rb[4];
+      // Interior tiles (every chunk complete and 16-byte aligned) take unconditional vector loads.
+      const bool fast = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
+      const T* wp[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        wp[i] = W_KC ? W + (int64_t)(c0 + (tid >> 3) + 32 * i) * p.w_snd + klo + a_chunk * CH
+                     : W + (int64_t)(klo + tid / CPR + RPP * i) * p.w_skd + c0 + (tid % CPR) * CH;
+      const int64_t w_step = W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd;
+      auto load_fast = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) ra[i] = *reinterpret_cast<const Raw*>(a_row[i] + klo + s * BK + a_chunk * CH);
+#pragma unroll
+        for (int i = 0; i < 4; i++) rb[i] = *reinterpret_cast<const Raw*>(wp[i] + s * w_step);
+      };
+      auto load_step = [&](int s) {          // global -> registers, any shape
+        const int k0 = klo + s * BK;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const int col = c0 + (tid >> 3) + 32 * i;
           const int kpos = k0 + a_chunk * CH;
-          int nv = col < c1 ? khi - kpos : 0;
+          int nv = a_ok[i] ? khi - kpos : 0;
           nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-          rb[i] = raw_load<T>(W + (int64_t)col * p.w_snd + kpos, nv, p.w_vec != 0);
+          ra[i] = raw_load<T>(a_row[i] + kpos, nv, p.a_vec != 0);
         }
-      } else {
+        if (W_KC) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int col = c0 + (tid >> 3) + 32 * i;
+            const int kpos = k0 + a_chunk * CH;
+            int nv = col < c1 ? khi - kpos : 0;
+            nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
+            rb[i] = raw_load<T>(W + (int64_t)col * p.w_snd + kpos, nv, p.w_vec != 0);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int kd = k0 + tid / CPR + RPP * i;
+            const int col = c0 + (tid % CPR) * CH;
+            int nv = kd < khi ? c1 - col : 0;
+            nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
+            rb[i] = raw_load<T>(W + (int64_t)kd * p.w_skd + col, nv, p.w_vec != 0);
+          }
+        }
+      };
+      auto store_step = [&](int buf) {       // registers -> LDS stage buf, DAC stage on the way
+        T* __restrict__ dA = sStage + buf * STAGE;
+        T* __restrict__ dB = dA + A_ELEMS;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const int kd = k0 + tid / CPR + RPP * i;
-          const int col = c0 + (tid % CPR) * CH;
-          int nv = kd < khi ? c1 - col : 0;
-          nv = nv < 0 ? 0 : (nv > CH ? CH : nv);
-          rb[i] = raw_load<T>(W + (int64_t)kd * p.w_skd + col, nv, p.w_vec != 0);
-        }
-      }
-    };
-    auto store_step = [&](int buf) {       // registers -> LDS stage buf, DAC stage on the way
-      T* __restrict__ dA = sA + buf * A_ELEMS;
-      T* __restrict__ dB = sB + buf * B_ELEMS;
+          Raw a = ra[i];
+          if (FWD && dac_ir_quant) {
+            float v[CH];
+            raw_unpack<T>(a, v);
+            const float r = a_ir[i], rinv = a_ir_inv[i];
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        Raw a = ra[i];
-        if (FWD && dac) {
-          float v[CH];
-          raw_unpack<T>(a, v);
-          bool out_of_range = false;
-#pragma unroll
-          for (int j = 0; j < CH; j++) {
-            float x = v[j];
-            if (has_ir) {
-              const float r = a_ir[i];
+            for (int j = 0; j < CH; j++) {
+              float x = v[j];
               x = x > r ? r : x;
               x = x < -r ? -r : x;
-              x = div_by(x, r, a_ir_inv[i]);
+              x = rintf(div_by(div_by(x, r, rinv), p.inp_res, inv_res));
+              v[j] = IS_BF16 ? x : x * p.inp_res;
             }
-            if (has_amax) x = div_by(x, a_amax[i], a_amax_inv[i]);
-            if (quant) {
-              out_of_range |= !(fabsf(x) <= 1.0f);
-              x = rintf(div_by(x, p.inp_res, inv_res));
-              if (!IS_BF16) x = x * p.inp_res;
+            if constexpr (IS_BF16) a = raw_pack_exact_bf16(v);
+            else a = raw_pack<T>(v);
+          } else if (FWD && dac) {
+            float v[CH];
+            raw_unpack<T>(a, v);
+            bool out_of_range = false;
+#pragma unroll
+            for (int j = 0; j < CH; j++) {
+              float x = v[j];
+              if (has_ir) {
+                const float r = a_ir[i];
+                x = x > r ? r : x;
+                x = x < -r ? -r : x;
+                x = div_by(x, r, a_ir_inv[i]);
+              }
+              if (has_amax) x = div_by(x, a_amax[i], a_amax_inv[i]);
+              if (quant) {
+                out_of_range |= !(fabsf(x) <= 1.0f);
+                x = rintf(div_by(x, p.inp_res, inv_res));
+                if (!IS_BF16) x = x * p.inp_res;
+              }
+              v[j] = x;
             }
-            v[j] = x;
+            if (quant && out_of_range && a_ok[i] && p.range_flag != nullptr) atomicOr(p.range_flag, 1);
+            if constexpr (IS_BF16) a = codes_mode ? raw_pack_exact_bf16(v) : raw_pack<T>(v);
+            else a = raw_pack<T>(v);
           }
-          if (quant && out_of_range && a_ok[i] && p.range_flag != nullptr) atomicOr(p.range_flag, 1);
-          if constexpr (IS_BF16) a = codes_mode ? raw_pack_exact_bf16(v) : raw_pack<T>(v);
-          else a = raw_pack<T>(v);
+          *reinterpret_cast<Raw*>(&dA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH]) = a;
+          if (W_KC) *reinterpret_cast<Raw*>(&dB[((tid >> 3) + 32 * i) * LDB + a_chunk * CH]) = rb[i];
+          else *reinterpret_cast<Raw*>(&dB[(tid / CPR + RPP * i) * LDB + (tid % CPR) * CH]) = rb[i];
         }
-        *reinterpret_cast<Raw*>(&dA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH]) = a;
-        if (W_KC) *reinterpret_cast<Raw*>(&dB[((tid >> 3) + 32 * i) * LDB + a_chunk * CH]) = rb[i];
-        else *reinterpret_cast<Raw*>(&dB[(tid / CPR + RPP * i) * LDB + (tid % CPR) * CH]) = rb[i];
-      }
-    };
+      };
 
-    if (fast) load_fast(0); else load_step(0);
-    store_step(0);
-    __syncthreads();
-    for (int s = 0; s < nsteps; s++) {
-      const int cur = s & 1;
-      if (s + 1 < nsteps) {                   // in flight while this stage is multiplied
-        if (fast) load_fast(s + 1); else load_step(s + 1);
+      if (fast) load_fast(0); else load_step(0);
+      store_step(0);
+      __syncthreads();
+      for (int s = 0; s < nsteps; s++) {
+        const int cur = s & 1;
+        if (s + 1 < nsteps) {                   // in flight while this stage is multiplied
+          if (fast) load_fast(s + 1); else load_step(s + 1);
+        }
+        const T* __restrict__ cA = sStage + cur * STAGE;
+        const T* __restrict__ cB = cA + A_ELEMS;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += MMAK) {
+          if constexpr (IS_BF16) {
+            u32x4 xf[2], wf[2];
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++)
+              xf[ti] = *reinterpret_cast<const u32x4*>(&cA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++) {
+              if (W_KC) {
+                wf[fi] = *reinterpret_cast<const u32x4*>(&cB[(wc * 64 + fi * 32 + l32) * LDB + kk + 8 * lh]);
+              } else {
+                const int R = lane & 15, g = (lane >> 4) & 1;
+                const uint16_t* base = reinterpret_cast<const uint16_t*>(
+                    &cB[(kk + 8 * lh + (R >> 2)) * LDB + wc * 64 + fi * 32 + 16 * g + 4 * (R & 3)]);
+                u32x2 lo = lds_read_tr16_b64(base);
+                u32x2 hi = lds_read_tr16_b64(base + 4 * LDB);
+                wf[fi] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+              }
+            }
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+              for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
+          } else {
+            float xf[2], wf[2];
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++) xf[ti] = cA[(wr * 64 + ti * 32 + l32) * LDA + kk + lh];
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++)
+              wf[fi] = W_KC ? cB[(wc * 64 + fi * 32 + l32) * LDB + kk + lh]
+                            : cB[(kk + lh) * LDB + wc * 64 + fi * 32 + l32];
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+              for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x2_f32(wf[fi], xf[ti], acc[fi][ti]);
+          }
+        }
+        if (s + 1 < nsteps) store_step(cur ^ 1);
+        __syncthreads();
       }
-      const T* __restrict__ cA = sA + cur * A_ELEMS;
-      const T* __restrict__ cB = sB + cur * B_ELEMS;
+
+      // ---- per-K-tile analog output stage (forward) ----------------------------------------------
+      if (FWD) {
+        const NoiseKey key = noise_key(p.seed, t);
 #pragma unroll
-      for (int kk = 0; kk < BK; kk += MMAK) {
-        if constexpr (IS_BF16) {
-          u32x4 xf[2], wf[2];
-#pragma unroll
-          for (int ti = 0; ti < 2; ti++)
-            xf[ti] = *reinterpret_cast<const u32x4*>(&cA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
+        for (int ti = 0; ti < 2; ti++) {
+          const int rl = wr * 64 + ti * 32 + l32;
+          const int r = row0 + rl;
+          const bool valid = r < row_end;
+          const int orow = valid ? sOrow[rl] : 0;
+          const float ir_r = (has_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
+          const float am_r = (has_amax && valid) ? p.abs_max[p.a_index[r]] : 1.f;
 #pragma unroll
           for (int fi = 0; fi < 2; fi++) {
-            if (W_KC) {
-              wf[fi] = *reinterpret_cast<const u32x4*>(&cB[(wc * 64 + fi * 32 + l32) * LDB + kk + 8 * lh]);
-            } else {
-              const int R = lane & 15, g = (lane >> 4) & 1;
-              const uint16_t* base = reinterpret_cast<const uint16_t*>(
-                  &cB[(kk + 8 * lh + (R >> 2)) * LDB + wc * 64 + fi * 32 + 16 * g + 4 * (R & 3)]);
-              u32x2 lo = lds_read_tr16_b64(base);
-              u32x2 hi = lds_read_tr16_b64(base + 4 * LDB);
-              wf[fi] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const int cl = wc * 64 + fi * 32 + 8 * q + 4 * lh;
+              const int col = c0 + cl;
+              int nv = valid ? c1 - col : 0;
+              nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+              float v[4];
+#pragma unroll
+              for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
+              if (codes_mode) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] *= p.inp_res;
+              }
+              if (p.noise != nullptr) {
+                float nz[4];
+                load4<float>(p.noise + (int64_t)t * p.noise_ts + (int64_t)orow * p.ldnoise + col, nz, nv,
+                             p.noise_vec != 0);
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] += nz[j];
+              } else if (gen_noise) {
+                float z[4];
+                const uint64_t ctr = (uint64_t)orow * (uint64_t)(p.ND >> 1) + (uint64_t)(col >> 1);
+                noise_pair(key, ctr, z[0], z[1]);
+                noise_pair(key, ctr + 1, z[2], z[3]);
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] += sCol[0][cl + j] * z[j];
+              }
+              if (adc_clip) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  const float b = sCol[1][cl + j];
+                  v[j] = fminf(fmaxf(v[j], -b), b);
+                  if (adc_quant) v[j] = rintf(v[j] * sCol[2][cl + j]) * sCol[3][cl + j];
+                }
+              }
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                if (has_amax) v[j] *= am_r;
+                if (has_ir) v[j] *= ir_r;
+                if (MODE == MODE_FWD_SPLIT) total[fi][ti][4 * q + j] += v[j];
+                else acc[fi][ti][4 * q + j] = v[j];
+              }
             }
           }
-#pragma unroll
-          for (int fi = 0; fi < 2; fi++)
-#pragma unroll
-            for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
-        } else {
-          float xf[2], wf[2];
-#pragma unroll
-          for (int ti = 0; ti < 2; ti++) xf[ti] = cA[(wr * 64 + ti * 32 + l32) * LDA + kk + lh];
-#pragma unroll
-          for (int fi = 0; fi < 2; fi++)
-            wf[fi] = W_KC ? cB[(wc * 64 + fi * 32 + l32) * LDB + kk + lh]
-                          : cB[(kk + lh) * LDB + wc * 64 + fi * 32 + l32];
-#pragma unroll
-          for (int fi = 0; fi < 2; fi++)
-#pragma unroll
-            for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x2_f32(wf[fi], xf[ti], acc[fi][ti]);
         }
       }
-      if (s + 1 < nsteps) store_step(cur ^ 1);
-      __syncthreads();
     }
 
-    // ---- per-K-tile analog output stage (forward) ------------------------------------------------
+    // ---- final values of the tile (in acc), then the store ------------------------------------
     if (FWD) {
-      const NoiseKey key = noise_key(p.seed, t);
+#pragma unroll
+      for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+        for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            float v = (MODE == MODE_FWD_SPLIT) ? total[fi][ti][i] : acc[fi][ti][i];
+            if (p.relu) v = v > 0.f ? v : 0.f;
+            acc[fi][ti][i] = v;
+          }
+    } else {
+      // input gradient: clip mask, input-range gradient partial sums, gate
+      const T* __restrict__ XF = static_cast<const T*>(p.xf);
+      const T* __restrict__ GATE = static_cast<const T*>(p.gate);
 #pragma unroll
       for (int ti = 0; ti < 2; ti++) {
-        const int r = row0 + wr * 64 + ti * 32 + l32;
+        const int rl = wr * 64 + ti * 32 + l32;
+        const int r = row0 + rl;
         const bool valid = r < row_end;
-        const int arow = valid ? p.a_index[r] : 0;
-        const int orow = valid ? (p.out_index ? p.out_index[r] : arow) : 0;
-        const float ir_r = (has_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
-        const float am_r = (has_amax && valid) ? p.abs_max[arow] : 1.f;
+        const int orow = valid ? sOrow[rl] : 0;
+        const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
+        const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
+        const float ir_r = (use_ir_bw && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile]
+                                                : 0.f;
+        float part = 0.f;
 #pragma unroll
         for (int fi = 0; fi < 2; fi++) {
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const int cl = wc * 64 + fi * 32 + 8 * q + 4 * lh;
-            const int col = c0 + cl;
+            const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
             int nv = valid ? c1 - col : 0;
+            nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+            float xv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, p.xf_vec != 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              float g = acc[fi][ti][4 * q + j];
+              if (j < nv) {
+                if (use_ir_bw) {
+                  const float gs = g * gate_r;
+                  if (xv[j] >= ir_r) part += fminf(gs, 0.f);
+                  if (xv[j] <= -ir_r) part -= fmaxf(gs, 0.f);
+                  const bool not_clip = fabsf(xv[j]) < ir_r;
+                  cnt += not_clip ? 1 : 0;
+                  g = not_clip ? g : 0.f;
+                }
+                if (p.relu_mask) g = xv[j] > 0.f ? g : 0.f;
+              }
+              acc[fi][ti][4 * q + j] = g * gate_r;
+            }
+          }
+        }
+        if (use_ir_bw) {
+          part += wave_shfl_xor(part, 32);
+          if (lh == 0) sRed[wc][rl] = part;
+        }
+      }
+    }
+
+    const bool staged = p.out_vec != 0 && (c1 - c0) == kTileCols;
+    if (staged) {
+      // registers -> LDS tile -> whole 256-byte (bf16) row segments to global memory
+      T* __restrict__ sOut = sStage;
+#pragma unroll
+      for (int h = 0; h < OUT_PASSES; h++) {
+        if (OUT_PASSES == 1 || wr == h) {
+#pragma unroll
+          for (int ti = 0; ti < 2; ti++) {
+            const int rl = (OUT_PASSES == 1 ? wr * 64 : 0) + ti * 32 + l32;
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
+                store4<T>(&sOut[rl * LDO + wc * 64 + fi * 32 + 8 * q + 4 * lh], v, 4, true);
+              }
+          }
+        }
+        __syncthreads();
+        constexpr int OCPR = kTileCols / CH;            // 16-byte chunks per row
+        constexpr int ORPP = kThreads / OCPR;
+#pragma unroll
+        for (int i = 0; i < OUT_ROWS / ORPP; i++) {
+          const int rl = tid / OCPR + ORPP * i;
+          const int orow = sOrow[h * OUT_ROWS + rl];
+          if (orow >= 0)
+            *reinterpret_cast<Raw*>(OUT + (int64_t)orow * p.ldo + c0 + (tid % OCPR) * CH) =
+                *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+        }
+        __syncthreads();
+      }
+    } else {
+#pragma unroll
+      for (int ti = 0; ti < 2; ti++) {
+        const int rl = wr * 64 + ti * 32 + l32;
+        const int orow = sOrow[rl];
+#pragma unroll
+        for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
+            int nv = orow >= 0 ? c1 - col : 0;
             nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
             float v[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
-            if (codes_mode) {
-#pragma unroll
-              for (int j = 0; j < 4; j++) v[j] *= p.inp_res;
-            }
-            if (p.noise != nullptr) {
-              float nz[4];
-              load4<float>(p.noise + (int64_t)t * p.noise_ts + (int64_t)orow * p.ldnoise + col, nz, nv,
-                           p.noise_vec != 0);
-#pragma unroll
-              for (int j = 0; j < 4; j++) v[j] += nz[j];
-            } else if (gen_noise) {
-              float z[4];
-              const uint64_t ctr = (uint64_t)orow * (uint64_t)(p.ND >> 1) + (uint64_t)(col >> 1);
-              noise_pair(key, ctr, z[0], z[1]);
-              noise_pair(key, ctr + 1, z[2], z[3]);
-#pragma unroll
-              for (int j = 0; j < 4; j++) v[j] += sCol[0][cl + j] * z[j];
-            }
-            if (adc_clip) {
-#pragma unroll
-              for (int j = 0; j < 4; j++) {
-                const float b = sCol[1][cl + j];
-                v[j] = fminf(fmaxf(v[j], -b), b);
-                if (adc_quant) v[j] = rintf(v[j] * sCol[2][cl + j]) * sCol[3][cl + j];
-              }
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-              if (has_amax) v[j] *= am_r;
-              if (has_ir) v[j] *= ir_r;
-              if (MODE == MODE_FWD_SPLIT) total[fi][ti][4 * q + j] += v[j];
-              else acc[fi][ti][4 * q + j] = v[j];
-            }
+            if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
           }
-        }
       }
+      __syncthreads();
+    }
+    if (use_ir_bw) {     // sRed was written before the barriers above
+      if (tid < kTileRows && row0 + tid < row_end)
+        p.irg_partial[(int64_t)cb * p.M + row0 + tid] = sRed[0][tid] + sRed[1][tid];
+      __syncthreads();
     }
   }
 
-  // ---- store ---------------------------------------------------------------------------------------
-  if (FWD) {
+  if (use_ir_bw) {
 #pragma unroll
-    for (int ti = 0; ti < 2; ti++) {
-      const int r = row0 + wr * 64 + ti * 32 + l32;
-      const bool valid = r < row_end;
-      const int orow = valid ? (p.out_index ? p.out_index[r] : p.a_index[r]) : 0;
-#pragma unroll
-      for (int fi = 0; fi < 2; fi++) {
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
-          int nv = valid ? c1 - col : 0;
-          nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
-          float v[4];
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            v[j] = (MODE == MODE_FWD_SPLIT) ? total[fi][ti][4 * q + j] : acc[fi][ti][4 * q + j];
-            if (p.relu) v[j] = v[j] > 0.f ? v[j] : 0.f;
-          }
-          if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
-        }
-      }
-    }
-  } else {
-    // ---- input gradient: clip mask, input-range gradient partial sums, gate ---------------------
-    const T* __restrict__ XF = static_cast<const T*>(p.xf);
-    const T* __restrict__ GATE = static_cast<const T*>(p.gate);
-    const bool use_ir = p.ir != nullptr;
-    int cnt = 0;
-#pragma unroll
-    for (int ti = 0; ti < 2; ti++) {
-      const int rl = wr * 64 + ti * 32 + l32;
-      const int r = row0 + rl;
-      const bool valid = r < row_end;
-      const int orow = valid ? p.out_index[r] : 0;
-      const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
-      const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
-      const float ir_r = (use_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile] : 0.f;
-      float part = 0.f;
-#pragma unroll
-      for (int fi = 0; fi < 2; fi++) {
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
-          int nv = valid ? c1 - col : 0;
-          nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
-          float v[4], xv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, p.xf_vec != 0);
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            float g = acc[fi][ti][4 * q + j];
-            if (j < nv) {
-              if (use_ir) {
-                const float gs = g * gate_r;
-                if (xv[j] >= ir_r) part += fminf(gs, 0.f);
-                if (xv[j] <= -ir_r) part -= fmaxf(gs, 0.f);
-                const bool not_clip = fabsf(xv[j]) < ir_r;
-                cnt += not_clip ? 1 : 0;
-                g = not_clip ? g : 0.f;
-              }
-              if (p.relu_mask) g = xv[j] > 0.f ? g : 0.f;
-            }
-            v[j] = g * gate_r;
-          }
-          if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
-        }
-      }
-      if (use_ir) {
-        part += wave_shfl_xor(part, 32);
-        if (lh == 0) sRed[wc][rl] = part;
-      }
-    }
-    if (use_ir) {
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) cnt += wave_shfl_xor(cnt, d);
-      if (lane == 0) sCnt[wave] = cnt;
-      __syncthreads();
-      if (tid < kTileRows && row0 + tid < row_end)
-        p.irg_partial[(int64_t)cb * p.M + row0 + tid] = sRed[0][tid] + sRed[1][tid];
-      if (tid == 0) p.notclip_count[lid] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
-    }
+    for (int d = 32; d >= 1; d >>= 1) cnt += wave_shfl_xor(cnt, d);
+    if (lane == 0) sCnt[wave] = cnt;
+    __syncthreads();
+    if (tid == 0) p.notclip_count[blockIdx.x] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
   }
 }
 

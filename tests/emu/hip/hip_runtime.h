@@ -33,6 +33,10 @@ typedef void* hipStream_t;
 enum { hipSuccess = 0 };
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emu"; }
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 0 };
+inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+// a 3-CU device: the persistent kernels then run few workgroups with several work items each
+inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 3; return hipSuccess; }
 
 struct EmuWave {
   std::barrier<> bar{64};
