@@ -42,13 +42,15 @@ inline int num_compute_units() {
 }
 
 // Persistent grid of the row-gather GEMM: two workgroups per compute unit, more if a workgroup
-// would otherwise own more row tiles than its descriptor table holds, never more than work items.
+// would otherwise get more work items than its descriptor table holds, rounded up to a multiple
+// of the column-block count (so that the column blocks of one row tile run side by side), never
+// more than there are work items.
 inline int persistent_grid(int row_tiles, int col_blocks) {
   const long long work = (long long)row_tiles * col_blocks;
   long long g = 2LL * num_compute_units();
-  const long long cap = (long long)(kMaxDesc - 2) * col_blocks;
-  const long long need = (work + cap - 1) / cap;
+  const long long need = (work + kMaxDesc - 1) / kMaxDesc;
   if (need > g) g = need;
+  if (g % col_blocks) g += col_blocks - g % col_blocks;
   if (g > work) g = work;
   return g < 1 ? 1 : (int)g;
 }

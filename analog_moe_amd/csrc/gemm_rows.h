@@ -52,9 +52,11 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int grid) {
 
 constexpr int kMaxDesc = 64;   // row tiles one workgroup can own (the host sizes the grid for it)
 
-// Persistent workgroups: the list of work items (row tile, column block), column block fastest,
-// is cut into gridDim.x contiguous ranges; a workgroup walks its range, keeping the row tile's
-// gather pointers while only the column block changes.
+// Persistent workgroups: the work items (row tile, column block), column block fastest, are dealt
+// round-robin to the workgroups (item w goes to logical workgroup w % gridDim.x).  Neighbouring
+// workgroups -- which the id remap keeps on one XCD -- therefore work on the column blocks of
+// the SAME row tile at the same time, so the gathered rows are read from HBM once and found in
+// that XCD's L2 by the others; the same holds for the weight tiles of consecutive row tiles.
 template <typename T, bool W_KC, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams p) {
   using EL = Elem<T>;
@@ -107,28 +109,27 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const int total_rt = sWave[0] + sWave[1] + sWave[2] + sWave[3];
   const int total_work = total_rt * ncb;
   const int lb = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int share = total_work / (int)gridDim.x, extra = total_work % (int)gridDim.x;
-  const int w0 = lb * share + (lb < extra ? lb : extra);
-  const int w1 = w0 + share + (lb < extra ? 1 : 0);
+  const int G = (int)gridDim.x;
+  const int n_my = lb < total_work ? (total_work - lb + G - 1) / G : 0;   // items lb, lb+G, ...
   int cnt = 0;                                       // un-clipped inputs seen by this lane (MODE_BWDX)
-  if (w0 < w1) {
-    const int rt_first = w0 / ncb, rt_last = (w1 - 1) / ncb;
-    // descriptors (expert, first sorted position, end position) of the row tiles of the range
+  {
+    // descriptors (expert, first sorted position, end position) of the row tiles of my items
     int t = tiles_before;
     for (int j = 0; j < per; j++) {
       const int e = e_first + j;
       if (e < p.E) {
         const int lo = p.offsets[e], hi = p.offsets[e + 1];
         const int nt = (hi - lo + kTileRows - 1) / kTileRows;
-        int a = rt_first > t ? rt_first : t;
-        const int b = rt_last < t + nt - 1 ? rt_last : t + nt - 1;
-        for (; a <= b; a++) {
-          const int slot = a - rt_first;
-          if (slot < kMaxDesc) {
-            const int r0 = lo + (a - t) * kTileRows;
-            sDesc[slot][0] = e;
-            sDesc[slot][1] = r0;
-            sDesc[slot][2] = r0 + kTileRows < hi ? r0 + kTileRows : hi;
+        if (nt > 0) {
+          // items whose row tile lies in [t, t+nt): w in [t*ncb, (t+nt)*ncb)
+          const int wlo = t * ncb, whi = (t + nt) * ncb;
+          int i = wlo > lb ? (wlo - lb + G - 1) / G : 0;
+          for (; i < n_my && i < kMaxDesc && lb + i * G < whi; i++) {
+            const int rt = (lb + i * G) / ncb;
+            const int r0 = lo + (rt - t) * kTileRows;
+            sDesc[i][0] = e;
+            sDesc[i][1] = r0;
+            sDesc[i][2] = r0 + kTileRows < hi ? r0 + kTileRows : hi;
           }
         }
         t += nt;
@@ -163,26 +164,40 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
   for (int i = 0; i < 4; i++) { a_row[i] = A; a_ok[i] = false; a_amax[i] = a_amax_inv[i] = 1.f; }
 
-  for (int w = w0; w < w1; w++) {
+  // row indices of the next item, fetched while the current one is multiplied
+  int n_idx[4] = {0, 0, 0, 0}, n_orow = -1;
+  auto fetch_rows = [&](int i) {
+    if (i >= n_my) return;
+    const int r0 = sDesc[i][1], r1 = sDesc[i][2];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int r = r0 + (tid >> 3) + 32 * q;
+      // rows past the tile read the tile's first row: safe to load, never stored
+      n_idx[q] = p.a_index[r < r1 ? r : r0];
+    }
+    if (tid < kTileRows) {
+      const int r = r0 + tid;
+      n_orow = r < r1 ? (p.out_index ? p.out_index[r] : p.a_index[r]) : -1;
+    }
+  };
+  fetch_rows(0);
+
+  for (int it = 0; it < n_my; it++) {
+    const int w = lb + it * G;
     const int rt = w / ncb, cb = w - rt * ncb;
-    if (rt != cur_rt) {                     // new row tile: gather pointers, scatter rows
+    {                                       // this item's row tile: gather pointers, scatter rows
       cur_rt = rt;
-      const int slot = rt - w0 / ncb;
-      e = sDesc[slot][0]; row0 = sDesc[slot][1]; row_end = sDesc[slot][2];
+      e = sDesc[it][0]; row0 = sDesc[it][1]; row_end = sDesc[it][2];
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int r = row0 + (tid >> 3) + 32 * i;
         a_ok[i] = r < row_end;
-        // rows past the tile read the tile's first row: safe to load, never stored
-        const int idx = p.a_index[a_ok[i] ? r : row0];
-        a_row[i] = A + (int64_t)idx * p.lda;
-        a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[idx] : 1.f;
+        a_row[i] = A + (int64_t)n_idx[i] * p.lda;
+        a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[n_idx[i]] : 1.f;
         a_amax_inv[i] = 1.0f / a_amax[i];
       }
-      if (tid < kTileRows) {
-        const int r = row0 + tid;
-        sOrow[tid] = r < row_end ? (p.out_index ? p.out_index[r] : p.a_index[r]) : -1;
-      }
+      if (tid < kTileRows) sOrow[tid] = n_orow;
+      fetch_rows(it + 1);
     }
     const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb);
     const int c0 = colb.c0, c1 = colb.c1;
