@@ -20,10 +20,7 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return as_f32((uint32_t)h << 16);
 }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = as_u32(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return (uint16_t)(pack_bf16x2(f, 0.f) & 0xffffu);   // hardware conversion, ties to even
 }
 
 // Element traits.  Chunk = 16 bytes of elements, the unit of global and LDS vector access.
@@ -133,8 +130,8 @@ __device__ __forceinline__ void store4(T* p, const float (&v)[4], int n_valid, b
       *reinterpret_cast<f32x4*>(p) = o;
     } else {
       u32x2 o;
-      o[0] = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-      o[1] = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+      o[0] = pack_bf16x2(v[0], v[1]);
+      o[1] = pack_bf16x2(v[2], v[3]);
       *reinterpret_cast<u32x2*>(p) = o;
     }
   } else {

@@ -151,6 +151,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
   const float inv_res = quant ? 1.0f / p.inp_res : 0.f;
   const bool use_ir_bw = !FWD && p.ir != nullptr;
+  // no analog output stage at all: the K-tile result is the accumulator itself
+  const bool plain_epi = !codes_mode && p.noise == nullptr && !gen_noise && !adc_clip && !has_amax && !has_ir;
 
   const int a_chunk = tid & 7;
   constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         a_ok[i] = r < row_end;
         a_row[i] = A + (int64_t)n_idx[i] * p.lda;
         a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[n_idx[i]] : 1.f;
-        a_amax_inv[i] = 1.0f / a_amax[i];
+        a_amax_inv[i] = has_amax ? 1.0f / a_amax[i] : 1.f;
       }
       if (tid < kTileRows) sOrow[tid] = n_orow;
       fetch_rows(it + 1);
@@ -235,7 +237,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       for (int i = 0; i < 4; i++) {
         const int r = row0 + (tid >> 3) + 32 * i;
         a_ir[i] = (has_ir && a_ok[i]) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
-        a_ir_inv[i] = 1.0f / a_ir[i];
+        a_ir_inv[i] = has_ir ? 1.0f / a_ir[i] : 1.f;
       }
 #pragma unroll
       for (int a = 0; a < 2; a++)
@@ -300,11 +302,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             const float r = a_ir[i], rinv = a_ir_inv[i];
 #pragma unroll
             for (int j = 0; j < CH; j++) {
-              float x = v[j];
-              x = x > r ? r : x;
-              x = x < -r ? -r : x;
-              x = rintf(div_by(div_by(x, r, rinv), p.inp_res, inv_res));
-              v[j] = IS_BF16 ? x : x * p.inp_res;
+              const float x = clamp_sym(v[j], r);
+              const float c = rintf(div_by(div_by(x, r, rinv), p.inp_res, inv_res));
+              v[j] = IS_BF16 ? c : c * p.inp_res;
             }
             if constexpr (IS_BF16) a = raw_pack_exact_bf16(v);
             else a = raw_pack<T>(v);
@@ -392,7 +392,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       }
 
       // ---- per-K-tile analog output stage (forward) ----------------------------------------------
-      if (FWD) {
+      if (FWD && plain_epi) {
+        if (MODE == MODE_FWD_SPLIT) {
+#pragma unroll
+          for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++) total[a][b] += acc[a][b];
+        }
+      } else if (FWD) {
         const NoiseKey key = noise_key(p.seed, t);
 #pragma unroll
         for (int ti = 0; ti < 2; ti++) {
@@ -454,16 +461,20 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 
     // ---- final values of the tile (in acc), then the store ------------------------------------
     if (FWD) {
+      if (MODE == MODE_FWD_SPLIT) {
 #pragma unroll
-      for (int fi = 0; fi < 2; fi++)
+        for (int fi = 0; fi < 2; fi++)
 #pragma unroll
-        for (int ti = 0; ti < 2; ti++)
+          for (int ti = 0; ti < 2; ti++) acc[fi][ti] = total[fi][ti];
+      }
+      if (p.relu) {
 #pragma unroll
-          for (int i = 0; i < 16; i++) {
-            float v = (MODE == MODE_FWD_SPLIT) ? total[fi][ti][i] : acc[fi][ti][i];
-            if (p.relu) v = v > 0.f ? v : 0.f;
-            acc[fi][ti][i] = v;
-          }
+        for (int fi = 0; fi < 2; fi++)
+#pragma unroll
+          for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[fi][ti][i] = fmaxf(acc[fi][ti][i], 0.f);
+      }
     } else {
       // input gradient: clip mask, input-range gradient partial sums, gate
       const T* __restrict__ XF = static_cast<const T*>(p.xf);

@@ -63,6 +63,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// clamp(x, -r, r) for r >= 0 as one v_med3_f32 (a NaN input gives -r or r instead of NaN).
+__device__ __forceinline__ float clamp_sym(float x, float r) { return __builtin_amdgcn_fmed3f(x, -r, r); }
+
 // sin / cos of 2*pi*x (x in revolutions), natural log, sqrt: single hardware instructions.
 __device__ __forceinline__ float fast_sin_rev(float x) { return __builtin_amdgcn_sinf(x); }
 __device__ __forceinline__ float fast_cos_rev(float x) { return __builtin_amdgcn_cosf(x); }

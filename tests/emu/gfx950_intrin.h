@@ -118,6 +118,7 @@ inline uint32_t emu_f32_to_bf16(float f) {
 }
 inline uint32_t pack_bf16x2(float lo, float hi) { return emu_f32_to_bf16(lo) | (emu_f32_to_bf16(hi) << 16); }
 
+inline float clamp_sym(float x, float r) { return x != x ? -r : (x > r ? r : (x < -r ? -r : x)); }
 inline float fast_sin_rev(float x) { return sinf(6.283185307179586f * x); }
 inline float fast_cos_rev(float x) { return cosf(6.283185307179586f * x); }
 inline float fast_log(float x) { return logf(x); }
