@@ -43,7 +43,7 @@ class BwdWArgs(C.Structure):
 class BwdXArgs(C.Structure):
     _fields_ = [
         ("dtype", C.c_int32), ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("E", C.c_int32),
-        ("g", P), ("ldg", C.c_int64),
+        ("g", P), ("ldg", C.c_int64), ("n_g_rows", C.c_int32),
         ("w", P), ("w_stride_e", C.c_int64), ("w_stride_k", C.c_int64),
         ("grad_x_full", P), ("ldo", C.c_int64),
         ("x", P), ("ldx", C.c_int64),

@@ -185,6 +185,9 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
                   : (a->w_stride_k % CH == 0));
   p.out_vec = aligned(a->out, 16) && (a->ldo % 4 == 0);
   p.noise_vec = a->noise && aligned(a->noise, 16) && (a->ldnoise % 4 == 0) && (a->noise_tile_stride % 4 == 0);
+  const long long lim = 1LL << 31;
+  p.buf_ok = (long long)a->n_in_rows * a->ldx * (long long)es < lim &&
+             ((long long)a->K * a->w_stride_k + (long long)a->N * a->w_stride_n) * (long long)es < lim;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -243,7 +246,7 @@ size_t amoe_bwd_x_workspace(int64_t M, int32_t K, int32_t n_tiles) {
 int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
   if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
-  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->E > kSelMaxExperts) return AMOE_EINVAL;
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->E > kSelMaxExperts || a->n_g_rows < 0) return AMOE_EINVAL;
   if (a->M == 0) return AMOE_OK;
   if (!a->g || !a->w || !a->grad_x_full || !a->offsets || !a->g_index || !a->out_index) return AMOE_ENULL;
   if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
@@ -278,6 +281,8 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   }
   p.a_vec = aligned(a->g, 16) && (a->ldg % CH == 0);
   p.w_vec = aligned(a->w, 16) && (a->w_stride_e % CH == 0) && (a->w_stride_k % CH == 0);
+  p.buf_ok = a->n_g_rows > 0 && (long long)a->n_g_rows * a->ldg * (long long)es < (1LL << 31) &&
+             (long long)a->K * a->w_stride_k * (long long)es < (1LL << 31);
   p.out_vec = aligned(a->grad_x_full, 16) && (a->ldo % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
   p.xf_vec = a->x && aligned(a->x, 16) && (a->ldx % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
   hipStream_t st = static_cast<hipStream_t>(stream);

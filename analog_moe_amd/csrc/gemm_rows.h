@@ -40,6 +40,7 @@ struct RowsParams {
   float* irg_partial; int32_t* notclip_count; int relu_mask;
   // vector-access permissions (alignment checked on the host)
   int a_vec, w_vec, out_vec, noise_vec, xf_vec;
+  int buf_ok;   // operands small enough for 32-bit byte offsets (buffer loads in the interior path)
 };
 
 // Workgroups are handed to the 8 XCDs round-robin; this maps the hardware id to a logical id so
@@ -161,10 +162,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   // state of the current row tile
   int e = 0, row0 = 0, row_end = 0, cur_rt = -1;
   const T* a_row[4];
+  uint32_t a_off[4];                      // byte offset of (row, chunk) from A, interior path
   bool a_ok[4];
   float a_amax[4], a_amax_inv[4];
 #pragma unroll
-  for (int i = 0; i < 4; i++) { a_row[i] = A; a_ok[i] = false; a_amax[i] = a_amax_inv[i] = 1.f; }
+  for (int i = 0; i < 4; i++) { a_row[i] = A; a_off[i] = 0; a_ok[i] = false; a_amax[i] = a_amax_inv[i] = 1.f; }
+  const BufRsrc rsrcA = make_rsrc(A);
 
   // row indices of the next item, fetched while the current one is multiplied
   int n_idx[4] = {0, 0, 0, 0}, n_orow = -1;
@@ -195,6 +198,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         const int r = row0 + (tid >> 3) + 32 * i;
         a_ok[i] = r < row_end;
         a_row[i] = A + (int64_t)n_idx[i] * p.lda;
+        a_off[i] = (uint32_t)(((int64_t)n_idx[i] * p.lda + a_chunk * CH) * (int64_t)sizeof(T));
         a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[n_idx[i]] : 1.f;
         a_amax_inv[i] = has_amax ? 1.0f / a_amax[i] : 1.f;
       }
@@ -248,18 +252,25 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 
       Raw ra[4], rb[4];
       // Interior tiles (every chunk complete and 16-byte aligned) take unconditional vector loads.
-      const bool fast = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
-      const T* wp[4];
+      const bool fast_shape = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
+      // the interior path addresses both operands with 32-bit byte offsets through buffer
+      // resources: per lane a fixed offset, per step a wave-uniform one
+      const bool fast = fast_shape && p.buf_ok != 0;
+      const BufRsrc rsrcW = make_rsrc(W);
+      uint32_t w_off[4];
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        wp[i] = W_KC ? W + (int64_t)(c0 + (tid >> 3) + 32 * i) * p.w_snd + klo + a_chunk * CH
-                     : W + (int64_t)(klo + tid / CPR + RPP * i) * p.w_skd + c0 + (tid % CPR) * CH;
-      const int64_t w_step = W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd;
+        w_off[i] = W_KC ? (uint32_t)((((int64_t)(c0 + (tid >> 3) + 32 * i)) * p.w_snd + a_chunk * CH) * (int64_t)sizeof(T))
+                        : (uint32_t)((((int64_t)(tid / CPR + RPP * i)) * p.w_skd + c0 + (tid % CPR) * CH) * (int64_t)sizeof(T));
+      const uint32_t a_step = BK * (uint32_t)sizeof(T);
+      const uint32_t w_step = (uint32_t)((W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd) * (int64_t)sizeof(T));
+      const uint32_t a_base = (uint32_t)klo * (uint32_t)sizeof(T);
+      const uint32_t w_base = (uint32_t)((W_KC ? (int64_t)klo : (int64_t)klo * p.w_skd) * (int64_t)sizeof(T));
       auto load_fast = [&](int s) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) ra[i] = *reinterpret_cast<const Raw*>(a_row[i] + klo + s * BK + a_chunk * CH);
+        for (int i = 0; i < 4; i++) ra[i] = buffer_load_b128(rsrcA, a_off[i], a_base + s * a_step);
 #pragma unroll
-        for (int i = 0; i < 4; i++) rb[i] = *reinterpret_cast<const Raw*>(wp[i] + s * w_step);
+        for (int i = 0; i < 4; i++) rb[i] = buffer_load_b128(rsrcW, w_off[i], w_base + s * w_step);
       };
       auto load_step = [&](int s) {          // global -> registers, any shape
         const int k0 = klo + s * BK;

@@ -38,6 +38,16 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(const uint16_t* p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
+// Raw buffer resource over [base, base + 4 GiB): loads take a per-lane 32-bit byte offset plus a
+// wave-uniform 32-bit byte offset, so the hot loops carry no 64-bit address arithmetic.
+typedef __amdgpu_buffer_rsrc_t BufRsrc;
+__device__ __forceinline__ BufRsrc make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buffer_load_b128(BufRsrc r, uint32_t lane_off, uint32_t uniform_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0);
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
 template <typename V>

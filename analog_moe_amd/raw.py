@@ -146,7 +146,7 @@ def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=No
     if g.shape[1] != N or grad_x_full.shape[1] != K:
         raise ValueError("g / w / grad_x_full shapes do not match")
     a.M, a.N, a.K, a.E = g_index.numel(), N, K, E
-    a.g, a.ldg = _p(g), g.stride(0)
+    a.g, a.ldg, a.n_g_rows = _p(g), g.stride(0), g.shape[0]
     a.w, a.w_stride_e, a.w_stride_k = _p(w), w.stride(0), w.stride(1)
     a.grad_x_full, a.ldo = _p(grad_x_full), grad_x_full.stride(0)
     if x is not None:

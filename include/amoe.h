@@ -150,7 +150,8 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* args, void* stream);
 typedef struct amoe_bwd_x_args {
   int32_t dtype;
   int32_t M, N, K, E;            /* as in the forward call: w is [E, K, N]; output has K columns */
-  const void* g;   int64_t ldg;  /* [*, N] */
+  const void* g;   int64_t ldg;  /* [n_g_rows, N] */
+  int32_t n_g_rows;
   const void* w;   int64_t w_stride_e, w_stride_k; /* [E, K, N], N contiguous */
   void* grad_x_full; int64_t ldo;   /* [n_out_rows, K] */
   const void* x;   int64_t ldx;  /* forward input [*, K]; may be NULL when ir == NULL and

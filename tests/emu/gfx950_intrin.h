@@ -11,6 +11,14 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
+typedef const unsigned char* BufRsrc;
+inline BufRsrc make_rsrc(const void* base) { return static_cast<const unsigned char*>(base); }
+inline u32x4 buffer_load_b128(BufRsrc r, uint32_t lane_off, uint32_t uniform_off) {
+  u32x4 v;
+  std::memcpy(&v, r + (size_t)lane_off + (size_t)uniform_off, 16);
+  return v;
+}
+
 inline int lane_id() { return threadIdx.x & 63; }
 
 template <class V> inline V emu_exchange(V v, int src) {
