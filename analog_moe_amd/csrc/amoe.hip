@@ -55,19 +55,39 @@ inline int persistent_grid(int row_tiles, int col_blocks) {
   return g < 1 ? 1 : (int)g;
 }
 
-template <typename T, bool W_KC>
-int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
+// Every tile of the launch is interior: the FAST instantiation applies.
+inline bool rows_all_interior(const RowsParams& p, int mode, int bk) {
+  if (!p.a_vec || !p.w_vec || !p.out_stage || !p.buf_ok || p.abs_max != nullptr) return false;
+  // forward: the edge-free code has the clip-and-quantise input stage or none at all
+  if (mode != MODE_BWDX && (p.ir != nullptr) != (p.inp_res > 0.f)) return false;
+  if (p.noise != nullptr && !p.noise_vec) return false;
+  if (p.xf != nullptr && !p.xf_vec) return false;
+  for (int t = 0; t < p.n_col_tiles; t++)
+    if ((p.col_bounds[t + 1] - p.col_bounds[t]) % kTileCols) return false;
+  for (int t = 0; t < p.n_kd_tiles; t++)
+    if ((p.kd_bounds[t + 1] - p.kd_bounds[t]) % bk) return false;
+  return true;
+}
+
+template <typename T, bool W_KC, bool FAST>
+int launch_rows_mode(const RowsParams& p, int mode, int grid, hipStream_t st) {
   if (mode == MODE_FWD) {
-    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD>;
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD, FAST>;
     hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
   } else if (mode == MODE_FWD_SPLIT) {
-    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD_SPLIT>;
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_FWD_SPLIT, FAST>;
     hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
   } else {
-    auto k = &gemm_rows_kernel<T, W_KC, MODE_BWDX>;
+    auto k = &gemm_rows_kernel<T, W_KC, MODE_BWDX, FAST>;
     hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
   }
   return launch_rc();
+}
+
+template <typename T, bool W_KC>
+int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
+  return rows_all_interior(p, mode, Elem<T>::kBK) ? launch_rows_mode<T, W_KC, true>(p, mode, grid, st)
+                                            : launch_rows_mode<T, W_KC, false>(p, mode, grid, st);
 }
 
 }  // namespace
@@ -119,7 +139,9 @@ int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, 
     hipLaunchKernelGGL(sel_hist_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
     if (int rc = launch_rc()) return rc;
   }
-  hipLaunchKernelGGL(sel_scan_kernel, dim3(1), dim3(kThreads), 0, st, p);
+  hipLaunchKernelGGL(sel_unit_scan_kernel, dim3((E + 3) / 4), dim3(kThreads), 0, st, p);
+  if (int rc = launch_rc()) return rc;
+  hipLaunchKernelGGL(sel_offsets_kernel, dim3(1), dim3(kThreads), 0, st, p);
   if (int rc = launch_rc()) return rc;
   if (blocks > 0) {
     hipLaunchKernelGGL(sel_scatter_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
@@ -184,6 +206,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
             (w_kc ? (a->w_stride_n % CH == 0 && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH))
                   : (a->w_stride_k % CH == 0));
   p.out_vec = aligned(a->out, 16) && (a->ldo % 4 == 0);
+  p.out_stage = aligned(a->out, 16) && (a->ldo % CH == 0);
   p.noise_vec = a->noise && aligned(a->noise, 16) && (a->ldnoise % 4 == 0) && (a->noise_tile_stride % 4 == 0);
   const long long lim = 1LL << 31;
   p.buf_ok = (long long)a->n_in_rows * a->ldx * (long long)es < lim &&
@@ -284,6 +307,7 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.buf_ok = a->n_g_rows > 0 && (long long)a->n_g_rows * a->ldg * (long long)es < (1LL << 31) &&
              (long long)a->K * a->w_stride_k * (long long)es < (1LL << 31);
   p.out_vec = aligned(a->grad_x_full, 16) && (a->ldo % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
+  p.out_stage = aligned(a->grad_x_full, 16) && (a->ldo % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   p.xf_vec = a->x && aligned(a->x, 16) && (a->ldx % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
   hipStream_t st = static_cast<hipStream_t>(stream);
   int rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
@@ -312,8 +336,9 @@ static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, 
   if (!z || !y) return AMOE_ENULL;
   const size_t es = esize(dtype);
   if (!aligned(z, es) || !aligned(y, es) || !aligned(gate, es)) return AMOE_EALIGN;
-  const int vec = aligned(z, 16) && aligned(y, 16) && (D % 4 == 0);
-  const long long work = (long long)T * ((D + 3) / 4);
+  const int CH = dtype == AMOE_F32 ? 4 : 8;
+  const int vec = aligned(z, 16) && aligned(y, 16) && (D % CH == 0);
+  const long long work = (long long)T * ((D + CH - 1) / CH);
   const long long blocks = (work + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -351,15 +376,16 @@ int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate
   const long long rows = (long long)T * k;
   const long long blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  const int vec = aligned(z, 16) && aligned(dy, 16) && (D % (dtype == AMOE_F32 ? 4 : 8) == 0);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == AMOE_F32) {
     auto kf = &gate_grad_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
-                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), rows, (int)k, (int)D);
+                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), rows, (int)k, (int)D, vec);
   } else {
     auto kf = &gate_grad_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
-                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), rows, (int)k, (int)D);
+                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), rows, (int)k, (int)D, vec);
   }
   return launch_rc();
 }
@@ -395,17 +421,18 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (cols == 1 || N == 1) {
     const long long per = (long long)K * N;
-    int chunks = (int)((per + 16 * kThreads - 1) / (16 * kThreads));
+    int chunks = (int)((per + 32 * kThreads - 1) / (32 * kThreads));
     chunks = chunks < 1 ? 1 : (chunks > 64 ? 64 : chunks);
+    const int vec = aligned(w, 16) && (per % 16 == 0);
     hipLaunchKernelGGL(fill_zero_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
                        reinterpret_cast<uint32_t*>(wmax), (int)E);
     if (int rc = launch_rc()) return rc;
     if (dtype == AMOE_F32) {
       auto kf = &weight_abs_max_kernel<float>;
-      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax, vec);
     } else {
       auto kf = &weight_abs_max_kernel<uint16_t>;
-      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax, vec);
     }
   } else {
     dim3 grid((N + kThreads - 1) / kThreads, E);

@@ -39,7 +39,7 @@ struct RowsParams {
   const void* xf; int64_t ldxf; const int32_t* xf_index; const void* gate;
   float* irg_partial; int32_t* notclip_count; int relu_mask;
   // vector-access permissions (alignment checked on the host)
-  int a_vec, w_vec, out_vec, noise_vec, xf_vec;
+  int a_vec, w_vec, out_vec, out_stage, noise_vec, xf_vec;   // out_stage: 16-byte row segments
   int buf_ok;   // operands small enough for 32-bit byte offsets (buffer loads in the interior path)
 };
 
@@ -58,7 +58,12 @@ constexpr int kMaxDesc = 64;   // row tiles one workgroup can own (the host size
 // workgroups -- which the id remap keeps on one XCD -- therefore work on the column blocks of
 // the SAME row tile at the same time, so the gathered rows are read from HBM once and found in
 // that XCD's L2 by the others; the same holds for the weight tiles of consecutive row tiles.
-template <typename T, bool W_KC, int MODE>
+//
+// FAST instantiations serve launches whose every tile is interior (the host checks: 16-byte
+// aligned operands, column tiles that are multiples of 128, K tiles that are multiples of the K
+// step, 32-bit addressable operands, no per-row abs-max scaling); they carry none of the
+// element-wise edge code.
+template <typename T, bool W_KC, int MODE, bool FAST>
 __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams p) {
   using EL = Elem<T>;
   constexpr int BK = EL::kBK, CH = EL::kChunk, MMAK = EL::kMmaK;
@@ -142,7 +147,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const T* __restrict__ A = static_cast<const T*>(p.a);
   T* __restrict__ OUT = static_cast<T*>(p.out);
   const bool has_ir = FWD && p.ir != nullptr;
-  const bool has_amax = FWD && p.abs_max != nullptr;
+  const bool has_amax = !FAST && FWD && p.abs_max != nullptr;
   const bool quant = FWD && p.inp_res > 0.f;
   const bool dac = has_ir || has_amax || quant;
   const bool dac_ir_quant = has_ir && quant && !has_amax;   // the common analog case: tight code
@@ -250,12 +255,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
           for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
 
-      Raw ra[4], rb[4];
+      Raw ra0[4], rb0[4];
       // Interior tiles (every chunk complete and 16-byte aligned) take unconditional vector loads.
       const bool fast_shape = p.a_vec != 0 && p.w_vec != 0 && (c1 - c0) == kTileCols && (khi - klo) % BK == 0;
       // the interior path addresses both operands with 32-bit byte offsets through buffer
       // resources: per lane a fixed offset, per step a wave-uniform one
-      const bool fast = fast_shape && p.buf_ok != 0;
+      const bool fast = FAST || (fast_shape && p.buf_ok != 0);
       const BufRsrc rsrcW = make_rsrc(W);
       uint32_t w_off[4];
 #pragma unroll
@@ -266,13 +271,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       const uint32_t w_step = (uint32_t)((W_KC ? (int64_t)BK : (int64_t)BK * p.w_skd) * (int64_t)sizeof(T));
       const uint32_t a_base = (uint32_t)klo * (uint32_t)sizeof(T);
       const uint32_t w_base = (uint32_t)((W_KC ? (int64_t)klo : (int64_t)klo * p.w_skd) * (int64_t)sizeof(T));
-      auto load_fast = [&](int s) {
+      auto load_fast = [&](int s, Raw (&ra)[4], Raw (&rb)[4]) {
 #pragma unroll
         for (int i = 0; i < 4; i++) ra[i] = buffer_load_b128(rsrcA, a_off[i], a_base + s * a_step);
 #pragma unroll
         for (int i = 0; i < 4; i++) rb[i] = buffer_load_b128(rsrcW, w_off[i], w_base + s * w_step);
       };
-      auto load_step = [&](int s) {          // global -> registers, any shape
+      auto load_step = [&](int s, Raw (&ra)[4], Raw (&rb)[4]) {   // global -> registers, any shape
         const int k0 = klo + s * BK;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -301,7 +306,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           }
         }
       };
-      auto store_step = [&](int buf) {       // registers -> LDS stage buf, DAC stage on the way
+      auto store_step = [&](int buf, Raw (&ra)[4], Raw (&rb)[4]) {   // registers -> LDS stage, DAC stage on the way
         T* __restrict__ dA = sStage + buf * STAGE;
         T* __restrict__ dB = dA + A_ELEMS;
 #pragma unroll
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             }
             if constexpr (IS_BF16) a = raw_pack_exact_bf16(v);
             else a = raw_pack<T>(v);
-          } else if (FWD && dac) {
+          } else if (!FAST && FWD && dac) {
             float v[CH];
             raw_unpack<T>(a, v);
             bool out_of_range = false;
@@ -350,14 +355,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         }
       };
 
-      if (fast) load_fast(0); else load_step(0);
-      store_step(0);
-      __syncthreads();
-      for (int s = 0; s < nsteps; s++) {
-        const int cur = s & 1;
-        if (s + 1 < nsteps) {                   // in flight while this stage is multiplied
-          if (fast) load_fast(s + 1); else load_step(s + 1);
+      auto load_any = [&](int s, Raw (&ra)[4], Raw (&rb)[4]) {
+        if constexpr (FAST) {
+          load_fast(s, ra, rb);
+        } else {
+          if (fast) load_fast(s, ra, rb); else load_step(s, ra, rb);
         }
+      };
+      auto multiply_stage = [&](int cur) {     // acc += stage `cur` of LDS
         const T* __restrict__ cA = sStage + cur * STAGE;
         const T* __restrict__ cB = cA + A_ELEMS;
 #pragma unroll
@@ -398,7 +403,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
               for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x2_f32(wf[fi], xf[ti], acc[fi][ti]);
           }
         }
-        if (s + 1 < nsteps) store_step(cur ^ 1);
+      };
+      load_any(0, ra0, rb0);
+      store_step(0, ra0, rb0);
+      __syncthreads();
+      for (int s = 0; s < nsteps; s++) {
+        if (s + 1 < nsteps) load_any(s + 1, ra0, rb0);
+        multiply_stage(s & 1);
+        if (s + 1 < nsteps) store_step((s + 1) & 1, ra0, rb0);
         __syncthreads();
       }
 
@@ -428,6 +440,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
               const int col = c0 + cl;
               int nv = valid ? c1 - col : 0;
               nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+              if (FAST) nv = valid ? 4 : 0;
               float v[4];
 #pragma unroll
               for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
@@ -438,7 +451,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
               if (p.noise != nullptr) {
                 float nz[4];
                 load4<float>(p.noise + (int64_t)t * p.noise_ts + (int64_t)orow * p.ldnoise + col, nz, nv,
-                             p.noise_vec != 0);
+                             FAST || p.noise_vec != 0);
 #pragma unroll
                 for (int j = 0; j < 4; j++) v[j] += nz[j];
               } else if (gen_noise) {
@@ -508,8 +521,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
             int nv = valid ? c1 - col : 0;
             nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+            if (FAST) nv = valid ? 4 : 0;
             float xv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, p.xf_vec != 0);
+            if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, FAST || p.xf_vec != 0);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
               float g = acc[fi][ti][4 * q + j];
@@ -535,7 +549,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       }
     }
 
-    const bool staged = p.out_vec != 0 && (c1 - c0) == kTileCols;
+    const bool staged = FAST || (p.out_stage != 0 && (c1 - c0) == kTileCols);
     if (staged) {
       // registers -> LDS tile -> whole 256-byte (bf16) row segments to global memory
       T* __restrict__ sOut = sStage;
@@ -569,7 +583,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         }
         __syncthreads();
       }
-    } else {
+    } else if constexpr (!FAST) {
 #pragma unroll
       for (int ti = 0; ti < 2; ti++) {
         const int rl = wr * 64 + ti * 32 + l32;

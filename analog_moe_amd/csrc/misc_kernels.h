@@ -6,39 +6,57 @@
 
 namespace amoe {
 
-// y[t, d] = sum_j gate[t*k+j] * z[(t*k+j), d]   (gate == nullptr: plain sum over j)
+// y[t, d] = sum_j gate[t*k+j] * z[(t*k+j), d]   (gate == nullptr: plain sum over j).
+// One thread per (row, 16-byte chunk); fp32 accumulation in ascending j.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restrict__ z, const T* __restrict__ gate,
                                                                 T* __restrict__ y, long long rows, int k, int D,
                                                                 int vec) {
-  const int quads = (D + 3) / 4;
+  constexpr int CH = Elem<T>::kChunk;
+  const int chunks = (D + CH - 1) / CH;
   const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
-  if (idx >= rows * quads) return;
-  const long long t = idx / quads;
-  const int d = (int)(idx % quads) * 4;
-  const int nv = D - d < 4 ? D - d : 4;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (idx >= rows * chunks) return;
+  const long long t = idx / chunks;
+  const int d = (int)(idx % chunks) * CH;
+  const int nv = D - d < CH ? D - d : CH;
+  float acc[CH];
+#pragma unroll
+  for (int q = 0; q < CH; q++) acc[q] = 0.f;
   for (int j = 0; j < k; j++) {
-    float v[4];
-    load4<T>(z + (t * k + j) * (long long)D + d, v, nv, vec != 0);
+    float v[CH];
+    raw_unpack<T>(raw_load<T>(z + (t * k + j) * (long long)D + d, nv, vec != 0), v);
     const float gt = gate ? Elem<T>::load(gate + t * k + j) : 1.f;
 #pragma unroll
-    for (int q = 0; q < 4; q++) acc[q] += gt * v[q];
+    for (int q = 0; q < CH; q++) acc[q] += gt * v[q];
   }
-  store4<T>(y + t * (long long)D + d, acc, nv, vec != 0);
+  T* out = y + t * (long long)D + d;
+  if (vec && nv == CH) {
+    *reinterpret_cast<Raw*>(out) = raw_pack<T>(acc);
+  } else {
+    for (int q = 0; q < nv; q++) out[q] = Elem<T>::cvt(acc[q]);
+  }
 }
 
-// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>, one wave per row.
+// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>, one wave per row, 16-byte chunks per lane.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict__ z, const T* __restrict__ dy,
-                                                              T* __restrict__ out, long long rows, int k, int D) {
+                                                              T* __restrict__ out, long long rows, int k, int D,
+                                                              int vec) {
+  constexpr int CH = Elem<T>::kChunk;
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   float s = 0.f;
   if (row < rows) {
     const T* zr = z + row * (long long)D;
     const T* dr = dy + (row / k) * (long long)D;
-    for (int d = lane; d < D; d += 64) s += Elem<T>::load(zr + d) * Elem<T>::load(dr + d);
+    for (int d = lane * CH; d < D; d += 64 * CH) {
+      const int nv = D - d < CH ? D - d : CH;
+      float a[CH], b[CH];
+      raw_unpack<T>(raw_load<T>(zr + d, nv, vec != 0), a);
+      raw_unpack<T>(raw_load<T>(dr + d, nv, vec != 0), b);
+#pragma unroll
+      for (int q = 0; q < CH; q++) s += a[q] * b[q];
+    }
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
@@ -79,15 +97,23 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restric
 }
 template <typename T>
 __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __restrict__ w, long long per_expert,
-                                                                   float* __restrict__ out) {
+                                                                   float* __restrict__ out, int vec) {
   __shared__ float red[4];
   const int tid = threadIdx.x, lane = tid & 63;
   const T* base = w + (long long)blockIdx.y * per_expert;
-  const long long span = (per_expert + gridDim.x - 1) / gridDim.x;
+  long long span = (per_expert + gridDim.x - 1) / gridDim.x;
+  span = (span + 15) / 16 * 16;             // keep slices 16-byte aligned
   const long long lo = (long long)blockIdx.x * span;
   const long long hi = lo + span < per_expert ? lo + span : per_expert;
+  constexpr int CH = Elem<T>::kChunk;
   float m = 0.f;
-  for (long long i = lo + tid; i < hi; i += kThreads) m = fmaxf(m, fabsf(Elem<T>::load(base + i)));
+  for (long long i = lo + (long long)tid * CH; i < hi; i += (long long)kThreads * CH) {
+    const int nv = hi - i < CH ? (int)(hi - i) : CH;
+    float v[CH];
+    raw_unpack<T>(raw_load<T>(base + i, nv, vec != 0), v);
+#pragma unroll
+    for (int q = 0; q < CH; q++) m = fmaxf(m, fabsf(v[q]));
+  }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, wave_shfl_xor(m, d));
   if (lane == 0) red[tid >> 6] = m;

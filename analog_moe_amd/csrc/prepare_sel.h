@@ -1,6 +1,7 @@
 // Expert sort of the CVMM path: stable counting sort of expert ids with wavefront ballots.
 //   pass 1  per-wave histograms of 1024-element units (LDS atomics)
-//   pass 2  one workgroup: per-expert totals -> offsets[E+1]; per-unit bases in place
+//   pass 2  a wave per expert scans its unit counts (bases in place), then one workgroup scans
+//           the per-expert totals -> offsets[E+1]
 //   pass 3  per wave: rank every element among equal keys of its 64-lane batch with a
 //           match-any built from ballots over the key bits, add the running per-key base kept
 //           in LDS, scatter (sorted id, flat index, flat index / k)
@@ -56,16 +57,40 @@ __global__ __launch_bounds__(kThreads) void sel_hist_kernel(const SelParams p) {
   }
 }
 
-__global__ __launch_bounds__(kThreads) void sel_scan_kernel(const SelParams p) {
+// pass 2a: one wave per expert turns its column of unit counts into unit bases relative to the
+// expert's segment start and writes the expert's total to offsets[e + 1].
+__global__ __launch_bounds__(kThreads) void sel_unit_scan_kernel(const SelParams p) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (e >= p.E) return;
+  int carry = 0;
+  for (int u0 = 0; u0 < p.n_units; u0 += 64) {
+    const int u = u0 + lane;
+    const int c = u < p.n_units ? p.unit_hist[(long long)u * p.E + e] : 0;
+    int incl = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = wave_shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (u < p.n_units) p.unit_hist[(long long)u * p.E + e] = carry + incl - c;
+    carry += wave_shfl(incl, 63);
+  }
+  if (lane == 0) p.offsets[e + 1] = carry;
+}
+
+// pass 2b: one workgroup turns the per-expert totals (in offsets[1..E]) into offsets[0..E].
+__global__ __launch_bounds__(kThreads) void sel_offsets_kernel(const SelParams p) {
+  constexpr int kPer = kSelMaxExperts / kThreads;
   __shared__ int wave_sums[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int per = (p.E + kThreads - 1) / kThreads;
-  const int e0 = tid * per;
+  const int e0 = tid * kPer;
+  int c[kPer];
   int mine = 0;
-  for (int j = 0; j < per; j++) {
-    const int e = e0 + j;
-    if (e < p.E)
-      for (int u = 0; u < p.n_units; u++) mine += p.unit_hist[(long long)u * p.E + e];
+#pragma unroll
+  for (int j = 0; j < kPer; j++) {
+    c[j] = e0 + j < p.E ? p.offsets[e0 + j + 1] : 0;
+    mine += c[j];
   }
   int incl = mine;
 #pragma unroll
@@ -74,20 +99,13 @@ __global__ __launch_bounds__(kThreads) void sel_scan_kernel(const SelParams p) {
     if (lane >= d) incl += up;
   }
   if (lane == 63) wave_sums[wave] = incl;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; w++) base += wave_sums[w];
-  int run = base + incl - mine;
-  for (int j = 0; j < per; j++) {
-    const int e = e0 + j;
-    if (e < p.E) {
-      p.offsets[e] = run;
-      for (int u = 0; u < p.n_units; u++) {
-        const int c = p.unit_hist[(long long)u * p.E + e];
-        p.unit_hist[(long long)u * p.E + e] = run;
-        run += c;
-      }
-    }
+  __syncthreads();                     // also orders every read of the totals before the writes below
+  int run = incl - mine;
+  for (int w = 0; w < wave; w++) run += wave_sums[w];
+#pragma unroll
+  for (int j = 0; j < kPer; j++) {
+    if (e0 + j < p.E) p.offsets[e0 + j] = run;
+    run += c[j];
   }
   if (tid == 0) p.offsets[p.E] = (int)p.M;
 }
@@ -98,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void sel_scatter_kernel(const SelParams p
   for (int w = 0; w < 4; w++) {
     const int u = blockIdx.x * 4 + w;
     if (u < p.n_units)
-      for (int e = tid; e < p.E; e += kThreads) base[w * p.E + e] = p.unit_hist[(long long)u * p.E + e];
+      for (int e = tid; e < p.E; e += kThreads) base[w * p.E + e] = p.offsets[e] + p.unit_hist[(long long)u * p.E + e];
   }
   __syncthreads();
   const int unit = blockIdx.x * 4 + wave;

@@ -33,7 +33,7 @@ def emu_ops():
     ops._LIB, ops._stream, ops._need_gpu = saved
 
 
-@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (66, 4, 2), (1500, 8, 2), (5000, 130, 4)])
+@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (66, 4, 2), (1500, 8, 2), (5000, 130, 4), (70000, 515, 3)])
 def test_prepare_sel_bit_exact(emu_ops, M, E, k):
     M -= M % k
     sel = torch.from_numpy(np.random.default_rng(M).integers(0, E, size=M))
@@ -62,6 +62,19 @@ CASES = {
                              dict(ir=True, inp_res=1 / 127, bounds_up=[0, 64, 128], out_bound=12.0, out_res=254.0,
                                   noise=0.04), "bf16", 2e-2),
     "f32_big_tile": (dict(T=200, D=40, E=2, F=136, k=2), dict(ir=True, inp_res=1 / 127), "f32", 1e-5),
+    # every tile interior: these run the edge-free instantiations of the row-gather GEMM
+    "f32_interior_split": (dict(T=80, D=128, E=3, F=128, k=2),
+                           dict(ir=True, inp_res=1 / 127, bounds_up=[0, 64, 128], bounds_down=[0, 32, 128],
+                                out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01), "f32", 1e-5),
+    "bf16_interior": (dict(T=80, D=128, E=3, F=128, k=2),
+                      dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01),
+                      "bf16", 2e-2),
+    "bf16_interior_split": (dict(T=80, D=128, E=3, F=256, k=2),
+                            dict(ir=True, inp_res=1 / 127, bounds_up=[0, 64, 128], bounds_down=[0, 128, 256],
+                                 out_bound=12.0, out_res=254.0, noise=0.04), "bf16", 2e-2),
+    "bf16_interior_plain": (dict(T=80, D=128, E=3, F=128, k=2), dict(), "bf16", 2e-2),
+    "f32_interior_ir_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(ir=True, decay=0.01), "f32", 1e-5),
+    "f32_interior_quant_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(inp_res=1 / 127), "f32", 1e-5),
 }
 
 
