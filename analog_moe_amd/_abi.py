@@ -23,7 +23,7 @@ class FwdArgs(C.Structure):
         ("ir", P), ("ir_by_expert", C.c_int32), ("abs_max", P), ("inp_res", C.c_float),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
         ("noise", P), ("noise_tile_stride", C.c_int64), ("ldnoise", C.c_int64),
-        ("noise_std", C.c_float), ("noise_seed", C.c_uint64),
+        ("noise_std", C.c_float), ("noise_seed", C.c_uint64), ("noise_seed_dev", C.c_void_p),
         ("wmax", P), ("wmax_cols", C.c_int32),
         ("out_bound", C.c_float), ("out_res", C.c_float),
         ("relu", C.c_int32), ("range_flag", P),

@@ -178,7 +178,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   const size_t es = esize(a->dtype);
   if (!aligned(a->x, es) || !aligned(a->w, es) || !aligned(a->out, es) || !aligned(a->offsets, 4) ||
       !aligned(a->in_index, 4) || !aligned(a->out_index, 4) || !aligned(a->ir, 4) || !aligned(a->abs_max, 4) ||
-      !aligned(a->noise, 4) || !aligned(a->wmax, 4) || !aligned(a->range_flag, 4))
+      !aligned(a->noise, 4) || !aligned(a->wmax, 4) || !aligned(a->range_flag, 4) || !aligned(a->noise_seed_dev, 8))
     return AMOE_EALIGN;
 
   const int CH = a->dtype == AMOE_F32 ? 4 : 8;
@@ -195,7 +195,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   p.ir = a->ir; p.ir_cols = a->n_tiles; p.ir_by_expert = a->ir_by_expert; p.abs_max = a->abs_max;
   p.inp_res = a->inp_res;
   p.noise = a->noise; p.noise_ts = a->noise_tile_stride; p.ldnoise = a->ldnoise;
-  p.noise_std = a->noise_std; p.seed = a->noise_seed;
+  p.noise_std = a->noise_std; p.seed = a->noise_seed; p.seed_dev = a->noise_seed_dev;
   p.wmax = a->wmax; p.wmax_cols = a->wmax_cols;
   p.out_bound = a->out_bound;
   p.out_half_states = (adc && a->out_res > 0.f) ? 0.5f * fmaxf(a->out_res, 1.0f / a->out_res) : 0.f;

@@ -32,7 +32,7 @@ struct RowsParams {
   int n_col_blocks;
   // forward
   const float* ir; int ir_cols; int ir_by_expert; const float* abs_max; float inp_res;
-  const float* noise; int64_t noise_ts, ldnoise; float noise_std; uint64_t seed;
+  const float* noise; int64_t noise_ts, ldnoise; float noise_std; uint64_t seed; const uint64_t* seed_dev;
   const float* wmax; int wmax_cols; float out_bound, out_half_states; int relu;
   int32_t* range_flag;
   // input gradient
@@ -155,6 +155,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const bool adc_clip = FWD && p.out_bound > 0.f;
   const bool adc_quant = adc_clip && p.out_half_states > 0.f;
   const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
+  const uint64_t seed = p.seed + ((gen_noise && p.seed_dev != nullptr) ? *p.seed_dev : 0);
   const float inv_res = quant ? 1.0f / p.inp_res : 0.f;
   const bool use_ir_bw = !FWD && p.ir != nullptr;
   // no analog output stage at all: the K-tile result is the accumulator itself
@@ -423,7 +424,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             for (int b = 0; b < 2; b++) total[a][b] += acc[a][b];
         }
       } else if (FWD) {
-        const NoiseKey key = noise_key(p.seed, t);
+        const NoiseKey key = noise_key(seed, t);
 #pragma unroll
         for (int ti = 0; ti < 2; ti++) {
           const int rl = wr * 64 + ti * 32 + l32;

@@ -62,6 +62,7 @@ class AnalogExt:
     out_res: float = -1.0
     noise_std: float = 0.0                       # generate noise in the kernel from noise_seed
     noise_seed: int = 0
+    noise_seed_dev: Optional[Tensor] = None      # int64 device word added to the seed by the kernel
 
 
 def _abs_max_wanted(ir_params, io_params) -> bool:
@@ -100,7 +101,7 @@ class CVMM(torch.autograd.Function):
             noise = out_noise.detach().float().reshape(n_tiles, M, N).contiguous()
         res = ops.cvmm_fwd(x, keys_op, ssel, offsets, sel_index, out_index, M, ir=bir, abs_max=abs_max,
                            inp_res=float(inp_res), bounds=ext.bounds, noise=noise, noise_std=ext.noise_std,
-                           noise_seed=ext.noise_seed, wmax=ext.wmax, out_bound=ext.out_bound,
+                           noise_seed=ext.noise_seed, noise_seed_dev=ext.noise_seed_dev, wmax=ext.wmax, out_bound=ext.out_bound,
                            out_res=ext.out_res)
         res = res.view(*sel.shape, N)
         z = None

@@ -25,6 +25,7 @@ class FFNConfig:
     out_res: float = -1.0
     noise_std: float = 0.0                        # in-kernel noise, in units of max|W|
     noise_seed: int = 0
+    noise_seed_dev: Optional[torch.Tensor] = None  # int64 device word added to the seed by the kernels
     noise_per_channel: bool = False
     gradient_relative: bool = True
     gradient_scale: float = 1.0
@@ -59,9 +60,11 @@ class AnalogMoEFFN(torch.autograd.Function):
         common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
                       noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
         p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, bounds=cfg.bounds_up,
-                          noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True, **common)
+                          noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True,
+                          noise_seed_dev=cfg.noise_seed_dev, **common)
         z = ops.cvmm_fwd(p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn, bounds=cfg.bounds_down,
-                         noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd, **common)
+                         noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
+                         noise_seed_dev=cfg.noise_seed_dev, **common)
         y = ops.gate_reduce(z, gate)
         ctx.save_for_backward(x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn)
         ctx.cfg = cfg

@@ -193,6 +193,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             raise MoEConifgError("noise_mode must be 'kernel' or 'injected'")
         self.noise_mode = noise_mode
         self._noise_calls = 0
+        self._init_done = False            # host-side latch of "input_range_update_idx reached init_from_data"
+        self.noise_counter: Optional[Tensor] = None     # see use_device_noise_counter()
         self._register_load_state_dict_pre_hook(load_state_dict_pre_hook)
         mis = getattr(self.rpu_config.mapping, "max_input_size", -1)
         self.bounds_up = tile_bounds(self.k_dim, mis)
@@ -294,9 +296,9 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         """Running average of init_std_alpha * std during the first init_from_data calls; one counter
         for both projections (moe_layer_aihwkit_lightning.py:432-445)."""
         ir_params = self.rpu_config.pre_post.input_range
-        idx = self.input_range_update_idx
-        if not (idx < ir_params.init_from_data):
+        if not self._init_from_data_pending():
             return
+        idx = self.input_range_update_idx
         stds = cvmm_std(inputs, sel_indices.sel_index, sel_indices.sel, self.n_experts).float()
         ok = stds > 0.0
         if ok.any():
@@ -306,7 +308,28 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             self.input_range_update_idx.data += 1
         self.input_range.data = self.input_range.data.abs()
 
+    def _init_from_data_pending(self) -> bool:
+        """True while the input ranges are still being initialised from data.  Costs no device
+        synchronisation when init_from_data is 0, and none after the initialisation has ended."""
+        n = self.rpu_config.pre_post.input_range.init_from_data
+        if n <= 0 or self._init_done:
+            return False
+        if not bool(self.input_range_update_idx < n):
+            self._init_done = True
+            return False
+        return True
+
+    def use_device_noise_counter(self) -> Tensor:
+        """Keep the per-call part of the noise seed in device memory (one int64 word that every noisy
+        launch reads and every forward bumps on the stream).  A forward captured in a HIP graph then
+        draws new noise on each replay; without it the seed is a launch argument frozen at capture."""
+        if self.noise_counter is None:
+            self.noise_counter = torch.zeros(1, dtype=torch.int64, device=self.keys.device)
+        return self.noise_counter
+
     def _noise_seed(self) -> int:
+        if self.noise_counter is not None:       # the call count lives on the device
+            return (torch.initial_seed() * 0x9E3779B97F4A7C15) & (2 ** 63 - 1)
         self._noise_calls += 1
         return (torch.initial_seed() * 0x9E3779B97F4A7C15 + self._noise_calls * 0xD1B54A32D192ED03) & (2 ** 63 - 1)
 
@@ -341,18 +364,22 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         out_noise = None
         if noisy and self.noise_mode == "kernel":
             ext.noise_std, ext.noise_seed = float(fwd.out_noise), self._noise_seed()
+            ext.noise_seed_dev = self.noise_counter
         elif noisy:
             shape = (nt, *sel_indices.raw_sel.shape, weights.shape[-1])
             out_noise = torch.randn(shape, device=inputs.device) * fwd.out_noise * ext.wmax[sel_indices.raw_sel]
-        return CVMM.apply(inputs, sel_indices.sel_index, sel_indices.sel, modified, inp_res, bir,
-                          sel_indices.out_index, sel_indices.reduction_weight, out_noise,
-                          self.rpu_config.pre_post.input_range, fwd, ext)
+        res = CVMM.apply(inputs, sel_indices.sel_index, sel_indices.sel, modified, inp_res, bir,
+                         sel_indices.out_index, sel_indices.reduction_weight, out_noise,
+                         self.rpu_config.pre_post.input_range, fwd, ext)
+        if ext.noise_seed_dev is not None:
+            ext.noise_seed_dev.add_(1)
+        return res
 
     # -- fused path ---------------------------------------------------------------------------------------
     def _fusable(self) -> bool:
         return (self.activation is F.relu and self.bias is None and self.dropout == 0 and
                 self.input_range is not None and enum_name(self.rpu_config.modifier.type) == "NONE" and
-                not (self.training and self.input_range_update_idx < self.rpu_config.pre_post.input_range.init_from_data))
+                not (self.training and self._init_from_data_pending()))
 
     def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
         if not x.is_cuda or not self._fusable():
@@ -363,6 +390,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         cfg = FFNConfig(inp_res=kernel_inp_res(fwd.inp_res), bounds_up=self.bounds_up, bounds_down=self.bounds_down,
                         out_bound=float(getattr(fwd, "out_bound", -1)), out_res=float(getattr(fwd, "out_res", -1)),
                         noise_std=float(fwd.out_noise) if noisy else 0.0, noise_seed=self._noise_seed() if noisy else 0,
+                        noise_seed_dev=self.noise_counter if noisy else None,
                         noise_per_channel=bool(getattr(fwd, "out_noise_per_channel", False)),
                         gradient_relative=getattr(irp, "gradient_relative", True),
                         gradient_scale=getattr(irp, "gradient_scale", 1.0), decay=irp.decay,
@@ -381,6 +409,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         y = AnalogMoEFFN.apply(x.reshape(-1, x.shape[-1]), self.keys.to(x.dtype), self.values.to(x.dtype),
                                self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
                                sel_idx.reshape(-1, self.n_heads), cfg)
+        if cfg.noise_seed_dev is not None:
+            cfg.noise_seed_dev.add_(2)             # the two projections used seed + 0 and seed + 1
         y = y.view(*lead, self.v_dim)
         if self.o_bias is not None:
             y = y + self.o_bias
@@ -397,6 +427,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
                                       error_msgs)
         if "rpu_config" in local_metadata:
             self.rpu_config = local_metadata["rpu_config"]
+        self._init_done = False
 
 
 # Names under which the reference exports its two flavours (analog_moe/__init__.py).

@@ -66,7 +66,7 @@ def offsets_from_sorted(lib, stream, sel_sorted, E: int, offsets):
 def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=None, ir=None, abs_max=None,
              inp_res: float = -1.0, bounds: Optional[Sequence[int]] = None, noise=None, noise_std: float = 0.0,
              noise_seed: int = 0, wmax=None, out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
-             range_flag=None, ir_by_expert: bool = False):
+             range_flag=None, ir_by_expert: bool = False, noise_seed_dev=None):
     """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N]."""
     _rows(x, "x"); _rows(out, "out")
     a = FwdArgs()
@@ -95,6 +95,10 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
             raise ValueError("noise must be [n_tiles, out rows, N]")
         a.noise, a.noise_tile_stride, a.ldnoise = _p(noise), out.shape[0] * N, N
     a.noise_std, a.noise_seed = float(noise_std), int(noise_seed) & 0xFFFFFFFFFFFFFFFF
+    if noise_seed_dev is not None:
+        if noise_seed_dev.dtype != torch.int64 or noise_seed_dev.numel() != 1:
+            raise ValueError("noise_seed_dev must be one int64 word")
+        a.noise_seed_dev = _p(noise_seed_dev)
     if wmax is not None:
         _f32(wmax, "wmax")
         a.wmax, a.wmax_cols = _p(wmax), wmax.numel() // E

@@ -33,6 +33,10 @@ CONFIGS = {
                name="config4: d_model=2048 E=128 F=512 k=4 32768 tokens bf16 Zipf(1.2) routing"),
 }
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
+# the counter runs summarised under profiles/; None where not measured
+TRAFFIC = {"c3": {"fwd_up": 427743943, "fwd_down": 465234679, "wgrad_down": 197429462, "wgrad_up": 194159204,
+                  "xgrad_down": 384312646, "xgrad_up": 683269889}}
 
 
 def cpu_baseline(cfg, pr, budget_tokens):
@@ -86,6 +90,9 @@ def main():
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=1024)
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run one 256 MiB device copy first (reference reading for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU hot path only; run it with --gpus 1", file=sys.stderr)
@@ -125,14 +132,22 @@ def main():
     dy = pr["dy"].to(dev)
     params = [layer.keys, layer.values, layer.input_range, x, gate]
 
+    layer.use_device_noise_counter()        # per-step noise seed in device memory: graph replays draw new noise
+
     def step():
         y = layer.forward_selected(x, gate, idx)
         y.backward(dy)
         for p in params:
             p.grad = None
 
-    # HIP events around every launch of the GEMM kernels, on the stream they are launched on
+    # HIP events around every launch, on the stream the kernels are launched on; a launch is named
+    # by its op and its position among that op's calls within one step
+    ROLES = {"cvmm_fwd": ["fwd_up (gemm_rows_kernel, forward, K-tile split)", "fwd_down (gemm_rows_kernel, forward)"],
+             "cvmm_bwd_w": ["wgrad_down (gemm_wgrad_kernel)", "wgrad_up (gemm_wgrad_kernel)"],
+             "cvmm_bwd_x": ["xgrad_down (gemm_rows_kernel, input gradient)",
+                            "xgrad_up (gemm_rows_kernel, input gradient)"]}
     events = {}
+    counter = {}
 
     def timed(name):
         fn = getattr(ops, name)
@@ -142,13 +157,26 @@ def main():
             s.record()
             r = fn(*a, **kw)
             e.record()
-            events.setdefault(name, []).append((s, e))
+            i = counter.get(name, 0)
+            counter[name] = i + 1
+            roles = ROLES.get(name)
+            key = roles[i % len(roles)] if roles else name
+            events.setdefault(key, []).append((s, e))
             return r
         return fn, wrapper
 
+    if args.copy_calibration:
+        # a plain device copy of known size: the scale for FETCH_SIZE / WRITE_SIZE readings of this run
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    # pass 1 (eager): HIP events around every launch give the per-launch durations
     saved = {}
     for name in ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x", "prepare_sel", "gate_reduce", "gate_grad", "ksum",
                  "weight_abs_max", "segment_sum"):
@@ -159,38 +187,62 @@ def main():
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    eager_ms = (time.perf_counter() - t0) / args.steps * 1e3
     for name, fn in saved.items():
         setattr(ops, name, fn)
 
+    # pass 2 (the headline): the same step captured once in a HIP graph and replayed; the launches
+    # are then back to back on the GPU instead of waiting for the Python that issues them
+    if args.no_graph:
+        elapsed = eager_ms * 1e-3 * args.steps
+    else:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+
     ms = elapsed / args.steps * 1e3
     M = T * k
-    flops_step = 12.0 * M * D * F                 # six GEMM passes of 2*M*D*F
+    flops_step = 12.0 * M * D * F                 # six GEMM launches of 2*M*D*F
     kern = {n: sum(s.elapsed_time(e) for s, e in ev) / len(ev) for n, ev in events.items()}
     calls = {n: len(ev) // args.steps for n, ev in events.items()}
     per_step = {n: kern[n] * calls[n] for n in kern}
-    gemms = ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x")
-    dom = max(gemms, key=lambda n: per_step[n])
+    gemms = [r for rs in ROLES.values() for r in rs if r in kern]
+    dom = max(gemms, key=lambda n: kern[n])       # the slowest single GEMM launch of a step
     gemm_flops = 2.0 * M * D * F                  # algorithmic flops of one launch of any of them
     achieved = gemm_flops / (kern[dom] * 1e-3)
     peak = PEAK[cfg["dtype"]]
+    traffic = TRAFFIC.get(args.config, {}).get(dom.split(" ")[0])
     out = {
         "metric": "analog MoE layer fwd+bwd tokens/sec on 1 GPU; % of MFMA peak TFLOP/s",
         "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms, "ms_per_step_eager": eager_ms, "launch": "eager" if args.no_graph else "hip graph replay",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["name"], "tokens": T, "d_model": D, "n_experts": E, "expert_size": F,
                    "top_k": k, "analog": "learned input range 3.0, 8-bit DAC, 8-bit ADC (out_bound 12), "
                    f"output noise {cfg['noise']} x max|W| drawn in-kernel, max_input_size {cfg['mis']}"},
         "tflops": flops_step / (ms * 1e-3) / 1e12,
         "pct_of_mfma_peak": 100.0 * flops_step / (ms * 1e-3) / peak,
-        "roofline": {"bound": "mfma", "kernel": {"cvmm_fwd": "gemm_rows_kernel (forward)",
-                                                  "cvmm_bwd_w": "gemm_wgrad_kernel",
-                                                  "cvmm_bwd_x": "gemm_rows_kernel (input gradient)"}[dom],
+        "roofline": {"bound": "mfma", "kernel": dom,
                      "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
-                     "frac": achieved / peak, "traffic": None,
+                     "frac": achieved / peak, "traffic": traffic,
                      "flops_per_launch": gemm_flops, "avg_launch_ms": kern[dom]},
-        "kernel_ms_per_step": {n: round(v, 4) for n, v in sorted(per_step.items(), key=lambda kv: -kv[1])},
+        "launch_ms": {n: round(v, 4) for n, v in sorted(kern.items(), key=lambda kv: -kv[1])},
+        "gemm_frac_of_peak": {n.split(" ")[0]: round(gemm_flops / (kern[n] * 1e-3) / peak, 4) for n in gemms},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, pr, args.cpu_tokens)

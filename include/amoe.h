@@ -97,6 +97,9 @@ typedef struct amoe_fwd_args {
   float noise_std;               /* used when noise == NULL and > 0: generate in the kernel
                                     noise_std * wmax[e, n] * N(0,1), N even */
   uint64_t noise_seed;
+  const uint64_t* noise_seed_dev;/* optional device word added to noise_seed when the kernel starts:
+                                    a captured graph draws new noise on each replay if the caller
+                                    bumps the word between replays */
   const float* wmax;             /* [E, wmax_cols] max |w| per expert (cols 1) or channel (N) */
   int32_t wmax_cols;
   float out_bound, out_res;      /* ADC: clamp to +-out_bound*wmax, max(res,1/res) states;

@@ -158,3 +158,73 @@ def test_input_range_init_from_data():
     std_up = O.expert_std(util.np32(x.reshape(-1, 128)), s.in_index, s.sel_sorted, 4)
     want_up = (2.0 * 0 + 3.0 * std_up) / 1                        # idx = 0 at the first call
     np.testing.assert_allclose(layer.input_range.data[0].cpu().numpy(), want_up, rtol=1e-4)
+
+
+def test_device_seed_word_is_added_to_the_seed():
+    """A launch with seed S and device word d draws the noise of a launch with seed S + d."""
+    from analog_moe_amd import ops
+    pr = util.make_problem(3, 64, 128, 4, 64, 2, dtype=torch.float32)
+    pr = {n: t.cuda() for n, t in pr.items()}
+    ss, perm, in_index, offsets = ops.prepare_sel(pr["idx"], 4, 2)
+    wmax = ops.weight_abs_max(pr["keys"], False)
+    kw = dict(noise_std=0.1, wmax=wmax)
+    word = torch.tensor([5], dtype=torch.int64, device="cuda")
+    a = ops.cvmm_fwd(pr["x"], pr["keys"], ss, offsets, in_index, perm, 128, noise_seed=100, noise_seed_dev=word, **kw)
+    b = ops.cvmm_fwd(pr["x"], pr["keys"], ss, offsets, in_index, perm, 128, noise_seed=105, **kw)
+    c = ops.cvmm_fwd(pr["x"], pr["keys"], ss, offsets, in_index, perm, 128, noise_seed=100, **kw)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+
+
+def test_layer_step_replays_from_a_hip_graph():
+    """Forward + backward of the noisy fused layer captured in a graph: every replay -- with eager work and
+    synchronisation between them -- equals the eager step run with the same value of the device seed word."""
+    from analog_moe_amd import config as cfgmod
+    layer = _layer(cfgmod, {}, d=128, E=4, F=128, k=2, dtype=torch.bfloat16, out_noise=0.04, out_bound=12.0,
+                   out_res=254, max_input_size=64, decay=0.01)
+    layer.train()
+    word = layer.use_device_noise_counter()
+    x = torch.randn(256, 128, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    sel_val, sel_idx, _ = layer.select(x.detach())
+    sel_val = sel_val.detach().requires_grad_()
+    dy = torch.randn(256, 128, device="cuda", dtype=torch.bfloat16)
+    params = [x, sel_val, layer.keys, layer.values, layer.input_range]
+
+    def step():
+        y = layer.forward_selected(x, sel_val, sel_idx)
+        y.backward(dy)
+        return y
+
+    def eager(at):
+        word.fill_(at)
+        for p in params:
+            p.grad = None
+        y = step()
+        return [y.detach().clone()] + [p.grad.clone() for p in params]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            eager(0)
+    torch.cuda.current_stream().wait_stream(side)
+    for p in params:
+        p.grad = None
+    word.fill_(0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_static = step()
+    outs = []
+    for r in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        outs.append([y_static.clone()] + [p.grad.clone() for p in params])
+        scratch = torch.randn(1 << 16, device="cuda").sum().item()      # eager work between replays
+        assert np.isfinite(scratch)
+    assert int(word.item()) == 6                                        # three replays bumped it by 2 each
+    saved = [p.grad for p in params]
+    for r in range(3):
+        want = eager(2 * r)
+        for g, w in zip(outs[r], want):
+            assert torch.equal(g, w)
+    assert not torch.equal(outs[0][0], outs[1][0])                      # new noise on every replay
+    del saved
