@@ -35,7 +35,7 @@ class BwdWArgs(C.Structure):
         ("dtype", C.c_int32), ("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("E", C.c_int32),
         ("x", P), ("ldx", C.c_int64), ("g", P), ("ldg", C.c_int64), ("grad_w", P),
         ("offsets", P), ("in_index", P), ("g_index", P), ("ir", P), ("ir_by_expert", C.c_int32),
-        ("g_scale", P),
+        ("g_scale", P), ("n_x_rows", C.c_int64), ("n_g_rows", C.c_int64),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
     ]
 

@@ -223,7 +223,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
 int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
   if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
-  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1) return AMOE_EINVAL;
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->n_x_rows < 0 || a->n_g_rows < 0) return AMOE_EINVAL;
   if (!a->grad_w || !a->offsets) return AMOE_ENULL;
   if (a->M > 0 && (!a->x || !a->g || !a->in_index)) return AMOE_ENULL;
   if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
@@ -244,6 +244,9 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   p.x_vec = aligned(a->x, 16) && (a->ldx % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   p.g_vec = aligned(a->g, 16) && (a->ldg % CH == 0);
   p.out_vec = aligned(a->grad_w, 16) && (a->N % 4 == 0);
+  p.out_stage = aligned(a->grad_w, 16) && (a->N % CH == 0);
+  p.buf_ok = a->n_x_rows > 0 && a->n_g_rows > 0 && a->n_x_rows * a->ldx * (long long)es < (1LL << 31) &&
+             a->n_g_rows * a->ldg * (long long)es < (1LL << 31);
   const long long grid = (long long)a->E * p.n_k_blocks * p.n_n_blocks;
   if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -5,6 +5,8 @@
 // Both operands are staged token-major ("RC": [token][feature], as they lie in memory) and
 // fed to the matrix unit through the transposing LDS read (bf16) or plain reads (fp32); the
 // gradient fragment is the A operand, so a lane holds one kk and runs of 4 consecutive n.
+// The clip and the optional per-row scale (the gate of the fused layer) are applied to the x
+// operand on its way into LDS; the finished tile leaves through LDS as whole row segments.
 #pragma once
 #include "common.h"
 #include "gemm_rows.h"
@@ -19,7 +21,8 @@ struct WgradParams {
   const int32_t* offsets; const int32_t* in_index; const int32_t* g_index;
   const float* ir; int ir_by_expert; const void* g_scale; int n_tiles; int bounds[kMaxTiles + 1];
   int n_k_blocks, n_n_blocks;
-  int x_vec, g_vec, out_vec;
+  int x_vec, g_vec, out_vec, out_stage;
+  int buf_ok;   // x and g small enough for 32-bit byte offsets (buffer loads on interior steps)
 };
 
 template <typename T>
@@ -33,8 +36,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   constexpr bool IS_BF16 = sizeof(T) == 2;
   static_assert(BT == 4 * RPP, "staging expects 4 passes");
 
-  __shared__ __attribute__((aligned(16))) T sX[2 * STAGE];   // two stages
-  __shared__ __attribute__((aligned(16))) T sG[2 * STAGE];
+  constexpr int LDO = kTileCols + 16 / (int)sizeof(T);       // staged output tile, rows of 128 + 16 bytes
+  static_assert(kTileRows * LDO <= 4 * STAGE, "the output tile must fit the stage buffers");
+  __shared__ __attribute__((aligned(16))) T sS[4 * STAGE];   // two stages of each operand
+  T* const sX = sS;
+  T* const sG = sS + 2 * STAGE;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave >> 1, wk = wave & 1;
@@ -64,90 +70,115 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][c][i] = 0.f;
 
-  // rows of the step after the one being loaded: indices are fetched one step ahead of the data
-  int nx_xi[4], nx_gi[4];
-  float nx_ir[4];
-  bool nx_ok[4];
-  auto load_index = [&](int i0) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int r = i0 + tid / CPR + RPP * i;
-      nx_ok[i] = r < seg1;
-      nx_xi[i] = nx_ok[i] ? p.in_index[r] : 0;
-      nx_gi[i] = nx_ok[i] ? (p.g_index ? p.g_index[r] : nx_xi[i]) : 0;
-      nx_ir[i] = (has_ir && !p.ir_by_expert && nx_ok[i]) ? p.ir[(int64_t)r * p.n_tiles + kcol.tile] : ir_expert;
-    }
+  // Per-row metadata of a step (x row, g row, scale, input range) is fetched by ONE lane per row
+  // and item -- thread group tid / BT picks the item -- two steps ahead of use, and handed to the
+  // other threads through the padding columns of the x stage rows: 16 bytes behind the 128
+  // operand columns of row j of a stage buffer.
+  auto meta = [&](int buf, int row) -> int* {
+    return reinterpret_cast<int*>(&sX[buf * STAGE + row * LD + kTileCols]);
   };
+  const int m_item = tid / BT, m_row = tid % BT;
+  int m_val = 0;
+  auto fetch_meta = [&](int i0) {            // global -> register, rows of the step that starts at i0
+    const int r = i0 + m_row;
+    const bool ok = r < seg1;
+    if (m_item == 0) m_val = ok ? p.in_index[r] : 0;
+    else if (m_item == 1) m_val = ok ? (p.g_index ? p.g_index[r] : p.in_index[r]) : 0;
+    else if (m_item == 2) m_val = (int)as_u32((GS != nullptr && ok) ? Elem<T>::load(GS + r) : 1.f);
+    else if (m_item == 3)
+      m_val = (int)as_u32((has_ir && !p.ir_by_expert && ok) ? p.ir[(int64_t)r * p.n_tiles + kcol.tile] : ir_expert);
+  };
+  auto publish_meta = [&](int buf) {
+    if (m_item < 4) meta(buf, m_row)[m_item] = m_val;
+  };
+
   Raw rx[4], rg[4];
-  float st_ir[4], st_gs[4];
-  auto load_step = [&]() {                   // global -> registers, rows from nx_*
+  auto load_step = [&](int i0, int mbuf) {   // global -> registers, any shape; rows from the metadata
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+      const int j = tid / CPR + RPP * i;
+      const bool ok = i0 + j < seg1;
+      const int* m = meta(mbuf, j);
       const int kk = kc0 + chunk * CH;
-      int nvx = nx_ok[i] ? kc1 - kk : 0;
+      int nvx = ok ? kc1 - kk : 0;
       nvx = nvx < 0 ? 0 : (nvx > CH ? CH : nvx);
-      rx[i] = raw_load<T>(X + (int64_t)nx_xi[i] * p.ldx + kk, nvx, p.x_vec != 0);
+      rx[i] = raw_load<T>(X + (int64_t)m[0] * p.ldx + kk, nvx, p.x_vec != 0);
       const int n = n0 + chunk * CH;
-      int nvg = nx_ok[i] ? n1 - n : 0;
+      int nvg = ok ? n1 - n : 0;
       nvg = nvg < 0 ? 0 : (nvg > CH ? CH : nvg);
-      rg[i] = raw_load<T>(G + (int64_t)nx_gi[i] * p.ldg + n, nvg, p.g_vec != 0);
-      st_ir[i] = nx_ir[i];
-      st_gs[i] = (GS != nullptr && nx_ok[i]) ? Elem<T>::load(GS + nx_xi[i]) : 1.f;
+      rg[i] = raw_load<T>(G + (int64_t)m[1] * p.ldg + n, nvg, p.g_vec != 0);
     }
   };
-  // Interior steps (all BT tokens exist, full 128-column tiles, aligned rows): unconditional loads.
-  const bool tile_fast = p.x_vec != 0 && p.g_vec != 0 && (kc1 - kc0) == kTileCols && (n1 - n0) == kTileCols;
-  auto load_fast = [&]() {
+  // Interior steps (all BT tokens exist, full 128-column tiles, aligned rows, 32-bit addressable
+  // operands): unconditional buffer loads, one 32-bit multiply per row address.
+  const bool tile_fast = p.x_vec != 0 && p.g_vec != 0 && p.buf_ok != 0 && (kc1 - kc0) == kTileCols &&
+                         (n1 - n0) == kTileCols;
+  const BufRsrc rsX = make_rsrc(X), rsG = make_rsrc(G);
+  const uint32_t x_row_bytes = (uint32_t)(p.ldx * (int64_t)sizeof(T)), g_row_bytes = (uint32_t)(p.ldg * (int64_t)sizeof(T));
+  const uint32_t x_col_bytes = (uint32_t)((kc0 + chunk * CH) * (int)sizeof(T));
+  const uint32_t g_col_bytes = (uint32_t)((n0 + chunk * CH) * (int)sizeof(T));
+  auto load_fast = [&](int mbuf) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      rx[i] = *reinterpret_cast<const Raw*>(X + (int64_t)nx_xi[i] * p.ldx + kc0 + chunk * CH);
-      rg[i] = *reinterpret_cast<const Raw*>(G + (int64_t)nx_gi[i] * p.ldg + n0 + chunk * CH);
-      st_ir[i] = nx_ir[i];
-      st_gs[i] = GS != nullptr ? Elem<T>::load(GS + nx_xi[i]) : 1.f;
+      const int* m = meta(mbuf, tid / CPR + RPP * i);
+      rx[i] = buffer_load_b128(rsX, (uint32_t)m[0] * x_row_bytes + x_col_bytes, 0);
+      rg[i] = buffer_load_b128(rsG, (uint32_t)m[1] * g_row_bytes + g_col_bytes, 0);
     }
   };
-  auto store_step = [&](int buf) {           // registers -> LDS, clip / gate scaling on the way
+  auto load_rows = [&](int i0, int mbuf) {
+    if (tile_fast && i0 + BT <= seg1) load_fast(mbuf); else load_step(i0, mbuf);
+  };
+  auto store_step = [&](int buf, int mbuf) {  // registers -> LDS, clip / row scaling of x on the way
     T* __restrict__ dX = sX + buf * STAGE;
     T* __restrict__ dG = sG + buf * STAGE;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      Raw x = rx[i], g = rg[i];
-      if (has_ir) {
+      const int j = tid / CPR + RPP * i;
+      Raw x = rx[i];
+      const Raw g = rg[i];
+      if (has_ir || GS != nullptr) {
+        const int* m = meta(mbuf, j);
+        const float scale = as_f32((uint32_t)m[2]), rng = as_f32((uint32_t)m[3]);
         float v[CH];
         raw_unpack<T>(x, v);
-        const float rng = st_ir[i];
+        if (has_ir) {
 #pragma unroll
-        for (int j = 0; j < CH; j++) {
-          v[j] = v[j] > rng ? rng : v[j];
-          v[j] = v[j] < -rng ? -rng : v[j];
+          for (int q = 0; q < CH; q++) v[q] = clamp_sym(v[q], rng);
+        }
+        if (GS != nullptr) {
+#pragma unroll
+          for (int q = 0; q < CH; q++) v[q] *= scale;
         }
         x = raw_pack<T>(v);
       }
-      if (GS != nullptr) {
-        float v[CH];
-        raw_unpack<T>(g, v);
-#pragma unroll
-        for (int j = 0; j < CH; j++) v[j] *= st_gs[i];
-        g = raw_pack<T>(v);
-      }
-      *reinterpret_cast<Raw*>(&dX[(tid / CPR + RPP * i) * LD + chunk * CH]) = x;
-      *reinterpret_cast<Raw*>(&dG[(tid / CPR + RPP * i) * LD + chunk * CH]) = g;
+      *reinterpret_cast<Raw*>(&dX[j * LD + chunk * CH]) = x;
+      *reinterpret_cast<Raw*>(&dG[j * LD + chunk * CH]) = g;
     }
   };
 
-  if (seg0 < seg1) {
-    load_index(seg0);
-    if (tile_fast && seg0 + BT <= seg1) load_fast(); else load_step();
-    load_index(seg0 + BT);
-    store_step(0);
+  // Pipeline, step s (rows seg0 + s*BT ...): data of step s is in stage s&1; the metadata of step
+  // s+1 sits in the padding of stage s&1 and that of step s+2 is published, at the end of step
+  // s, into the padding of stage (s+1)&1 together with the data of step s+1.
+  const int nsteps = (seg1 - seg0 + BT - 1) / BT;
+  if (nsteps > 0) {
+    fetch_meta(seg0);
+    publish_meta(1);                          // metadata of step 0, parked in stage 1
+    __syncthreads();
+    load_rows(seg0, 1);
+    fetch_meta(seg0 + BT);
+    __syncthreads();                          // every thread has read its step-0 metadata
+    // (the scale / range of step 0 are still in stage 1's padding, which nothing has overwritten)
+    store_step(0, 1);
+    __syncthreads();                          // ... before the metadata of step 1 replaces it
+    publish_meta(0);
+    __syncthreads();
   }
-  __syncthreads();
-  int cur = 0;
-  for (int i0 = seg0; i0 < seg1; i0 += BT) {
-    const bool more = i0 + BT < seg1;
+  for (int s = 0; s < nsteps; s++) {
+    const int cur = s & 1;
+    const bool more = s + 1 < nsteps;
     if (more) {
-      if (tile_fast && i0 + 2 * BT <= seg1) load_fast(); else load_step();
-      load_index(i0 + 2 * BT);
+      load_rows(seg0 + (s + 1) * BT, cur);    // rows of step s+1: metadata in stage cur's padding
+      fetch_meta(seg0 + (s + 2) * BT);
     }
     const T* __restrict__ cX = sX + cur * STAGE;
     const T* __restrict__ cG = sG + cur * STAGE;
@@ -183,12 +214,41 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
           for (int fk = 0; fk < 2; fk++) acc[fn][fk] = mfma_32x32x2_f32(gf[fn], xf[fk], acc[fn][fk]);
       }
     }
-    if (more) store_step(cur ^ 1);
+    if (more) {
+      // the scale / range of step s+1 are read from stage cur's padding; the metadata of step
+      // s+2 goes to the padding of the stage that receives the data of step s+1
+      store_step(cur ^ 1, cur);
+      publish_meta(cur ^ 1);
+    }
     __syncthreads();
-    cur ^= 1;
   }
 
   T* __restrict__ GW = static_cast<T*>(p.grad_w) + (int64_t)e * p.K * p.N;
+  if (p.out_stage != 0 && (kc1 - kc0) == kTileCols && (n1 - n0) == kTileCols) {
+    // registers -> LDS tile -> whole 256-byte (bf16) / 512-byte (fp32) row segments.  The barrier
+    // that ended the last step has retired every read of the stage buffers.
+    T* __restrict__ sOut = sS;
+#pragma unroll
+    for (int fk = 0; fk < 2; fk++)
+#pragma unroll
+      for (int fn = 0; fn < 2; fn++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; j++) v[j] = acc[fn][fk][4 * q + j];
+          store4<T>(&sOut[(wk * 64 + fk * 32 + l32) * LDO + wn * 64 + fn * 32 + 8 * q + 4 * lh], v, 4, true);
+        }
+    __syncthreads();
+    constexpr int OCPR = kTileCols / CH, ORPP = kThreads / OCPR;
+#pragma unroll
+    for (int i = 0; i < kTileRows / ORPP; i++) {
+      const int rl = tid / OCPR + ORPP * i;
+      *reinterpret_cast<Raw*>(GW + (int64_t)(kc0 + rl) * p.N + n0 + (tid % OCPR) * CH) =
+          *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+    }
+    return;
+  }
 #pragma unroll
   for (int fk = 0; fk < 2; fk++) {
     const int kk = kc0 + wk * 64 + fk * 32 + l32;

@@ -118,7 +118,8 @@ def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.
     _need_gpu(x, g, offsets, in_index, g_index, ir, g_scale)
     x2, g2 = _rows2d(x), _rows2d(g)
     grad_w = torch.empty((n_experts, x2.shape[1], g2.shape[1]), dtype=x2.dtype, device=x2.device)
-    gs = None if g_scale is None else g_scale.detach().reshape(-1).to(x2.dtype).contiguous()
+    # the library wants the scale per sorted position
+    gs = None if g_scale is None else g_scale.detach().reshape(-1).to(x2.dtype)[in_index.long()].contiguous()
     raw.cvmm_bwd_w(get_lib(), _stream(x2), x2, g2, grad_w, offsets, in_index, g_index, _f32c(ir), bounds,
                    ir_by_expert, gs)
     return grad_w

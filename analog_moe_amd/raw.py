@@ -129,6 +129,7 @@ def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=No
     if g_scale is not None and (g_scale.dtype != x.dtype or not g_scale.is_contiguous()):
         raise TypeError("g_scale must be contiguous and share the dtype of x")
     a.g_scale = _p(g_scale)
+    a.n_x_rows, a.n_g_rows = x.shape[0], g.shape[0]
     check(lib, lib.amoe_cvmm_bwd_w(C.byref(a), stream), "amoe_cvmm_bwd_w")
 
 

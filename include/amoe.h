@@ -129,10 +129,12 @@ typedef struct amoe_bwd_w_args {
                                             (cvmm.py:346-351) */
   const float* ir;                       /* [M, n_tiles] or NULL */
   int32_t ir_by_expert;                  /* != 0: ir is [E, n_tiles] */
-  const void* g_scale;                   /* dtype, indexed by in_index[i], or NULL: the g row is
-                                            multiplied by it and rounded to dtype, which is the
-                                            gate (x) dy outer product of cvmm.py:785-789 without
-                                            materialising it */
+  const void* g_scale;                   /* dtype, [M], one value per sorted position, or NULL: the
+                                            clipped x row is multiplied by it and rounded to dtype, which
+                                            gives the gate (x) dy outer product of cvmm.py:785-789
+                                            without materialising it */
+  int64_t n_x_rows, n_g_rows;            /* rows of x and of g (bounds the 32-bit addressing of the
+                                            interior path; 0 = unknown: 64-bit addressing) */
   int32_t n_tiles;
   int32_t tile_bounds[AMOE_MAX_TILES + 1];
 } amoe_bwd_w_args;
