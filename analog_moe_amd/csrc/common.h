@@ -252,7 +252,7 @@ __device__ __forceinline__ void noise_pair(const NoiseKey& key, uint64_t pair_ct
   h ^= h >> 16; h *= 0x85EBCA6Bu; h += key.kb; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
   float u1 = ((float)(h >> 16) + 0.5f) * (1.0f / 65536.0f);
   float u2 = ((float)(h & 0xffffu) + 0.5f) * (1.0f / 65536.0f);
-  float r = fast_sqrt(-2.0f * fast_log(u1));
+  float r = fast_sqrt(-1.3862943611f * fast_log2(u1));     // sqrt(-2 ln u1)
   z0 = r * fast_cos_rev(u2);
   z1 = r * fast_sin_rev(u2);
 }

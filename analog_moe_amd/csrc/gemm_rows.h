@@ -78,12 +78,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   constexpr int LDO = kTileCols + 16 / (int)sizeof(T);
   constexpr int OUT_PASSES = IS_BF16 ? 1 : 2;
   constexpr int OUT_ROWS = kTileRows / OUT_PASSES;
-  static_assert(OUT_ROWS * LDO <= 2 * STAGE, "output staging must fit the stage buffers");
+  static_assert(OUT_ROWS * LDO <= (IS_BF16 ? STAGE : 2 * STAGE), "output staging must fit the stage buffers");
 
   __shared__ __attribute__((aligned(16))) T sStage[2 * STAGE];
   __shared__ __attribute__((aligned(16))) float sCol[4][kTileCols];
   __shared__ float sRed[2][kTileRows];
   __shared__ int sOrow[kTileRows];
+  __shared__ int sXrow[kTileRows];                // rows of the forward input of the tile (MODE_BWDX)
   __shared__ int sDesc[kMaxDesc][4];
   __shared__ int sCnt[4];
   __shared__ int sWave[4];
@@ -176,7 +177,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const BufRsrc rsrcA = make_rsrc(A);
 
   // row indices of the next item, fetched while the current one is multiplied
-  int n_idx[4] = {0, 0, 0, 0}, n_orow = -1;
+  int n_idx[4] = {0, 0, 0, 0}, n_orow = -1, n_xrow = 0;
+  // input gradient, bf16, edge-free: the forward-input tile behind the clip / ReLU masks is read as
+  // whole row segments during the last K step and handed to the epilogue through LDS
+  const bool xf_stage = FAST && IS_BF16 && !FWD && p.xf != nullptr;
   auto fetch_rows = [&](int i) {
     if (i >= n_my) return;
     const int r0 = sDesc[i][1], r1 = sDesc[i][2];
@@ -189,6 +193,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
     if (tid < kTileRows) {
       const int r = r0 + tid;
       n_orow = r < r1 ? (p.out_index ? p.out_index[r] : p.a_index[r]) : -1;
+      if (xf_stage) n_xrow = p.xf_index[r < r1 ? r : r0];
     }
   };
   fetch_rows(0);
@@ -208,7 +213,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         a_amax[i] = (has_amax && a_ok[i]) ? p.abs_max[n_idx[i]] : 1.f;
         a_amax_inv[i] = has_amax ? 1.0f / a_amax[i] : 1.f;
       }
-      if (tid < kTileRows) sOrow[tid] = n_orow;
+      if (tid < kTileRows) {
+        sOrow[tid] = n_orow;
+        if (xf_stage) sXrow[tid] = n_xrow;
+      }
       fetch_rows(it + 1);
     }
     const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb);
@@ -409,9 +417,26 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       store_step(0, ra0, rb0);
       __syncthreads();
       for (int s = 0; s < nsteps; s++) {
-        if (s + 1 < nsteps) load_any(s + 1, ra0, rb0);
+        if (s + 1 < nsteps) {
+          load_any(s + 1, ra0, rb0);
+        } else if (xf_stage) {                // last step: the staging registers fetch the mask tile
+          const T* __restrict__ XF = static_cast<const T*>(p.xf);
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            const int rl = tid / 16 + 16 * i;
+            const Raw v = *reinterpret_cast<const Raw*>(XF + (int64_t)sXrow[rl] * p.ldxf + c0 + (tid % 16) * CH);
+            if (i < 4) ra0[i] = v; else rb0[i - 4] = v;
+          }
+        }
         multiply_stage(s & 1);
-        if (s + 1 < nsteps) store_step((s + 1) & 1, ra0, rb0);
+        if (s + 1 < nsteps) {
+          store_step((s + 1) & 1, ra0, rb0);
+        } else if (xf_stage) {                // ... and park it in the stage that is idle now
+          T* __restrict__ sXF = sStage + ((s + 1) & 1) * STAGE;
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+            *reinterpret_cast<Raw*>(&sXF[(tid / 16 + 16 * i) * LDO + (tid % 16) * CH]) = i < 4 ? ra0[i] : rb0[i - 4];
+        }
         __syncthreads();
       }
 
@@ -510,7 +535,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         const int r = row0 + rl;
         const bool valid = r < row_end;
         const int orow = valid ? sOrow[rl] : 0;
-        const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
+        const int xrow = (valid && XF != nullptr && !xf_stage) ? p.xf_index[r] : 0;
         const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
         const float ir_r = (use_ir_bw && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile]
                                                 : 0.f;
@@ -524,7 +549,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
             if (FAST) nv = valid ? 4 : 0;
             float xv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (XF != nullptr && nv > 0) load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, FAST || p.xf_vec != 0);
+            if (xf_stage) {
+              const int nst = (p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK;
+              load4<T>(&sStage[(nst & 1) * STAGE + rl * LDO + col - c0], xv, 4, true);
+            } else if (XF != nullptr && nv > 0) {
+              load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, FAST || p.xf_vec != 0);
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
               float g = acc[fi][ti][4 * q + j];
@@ -553,7 +583,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
     const bool staged = FAST || (p.out_stage != 0 && (c1 - c0) == kTileCols);
     if (staged) {
       // registers -> LDS tile -> whole 256-byte (bf16) row segments to global memory
-      T* __restrict__ sOut = sStage;
+      // (the input gradient may still be reading the parked mask tile from the other stage)
+      T* __restrict__ sOut = sStage + ((!FWD && ((p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK) % 2 == 0) ? STAGE : 0);
 #pragma unroll
       for (int h = 0; h < OUT_PASSES; h++) {
         if (OUT_PASSES == 1 || wr == h) {

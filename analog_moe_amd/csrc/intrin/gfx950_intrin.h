@@ -79,7 +79,8 @@ __device__ __forceinline__ float clamp_sym(float x, float r) { return __builtin_
 // sin / cos of 2*pi*x (x in revolutions), natural log, sqrt: single hardware instructions.
 __device__ __forceinline__ float fast_sin_rev(float x) { return __builtin_amdgcn_sinf(x); }
 __device__ __forceinline__ float fast_cos_rev(float x) { return __builtin_amdgcn_cosf(x); }
-__device__ __forceinline__ float fast_log(float x) { return __logf(x); }
+// log2 of a normal positive number (no denormal handling)
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 __device__ __forceinline__ uint32_t umulhi32(uint32_t a, uint32_t b) { return __umulhi(a, b); }
 
