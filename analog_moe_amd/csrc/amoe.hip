@@ -247,7 +247,7 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   p.out_stage = aligned(a->grad_w, 16) && (a->N % CH == 0);
   p.buf_ok = a->n_x_rows > 0 && a->n_g_rows > 0 && a->n_x_rows * a->ldx * (long long)es < (1LL << 31) &&
              a->n_g_rows * a->ldg * (long long)es < (1LL << 31);
-  const long long grid = (long long)a->E * p.n_k_blocks * p.n_n_blocks;
+  const long long grid = 8LL * ((a->E + 7) / 8) * p.n_k_blocks * p.n_n_blocks;   // see the id mapping in the kernel
   if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (a->dtype == AMOE_F32) {

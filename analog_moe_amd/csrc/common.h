@@ -62,6 +62,19 @@ __device__ __forceinline__ Raw raw_load(const T* p, int n_valid, bool vec) {
   if (vec && n_valid >= C) return *reinterpret_cast<const Raw*>(p);
   Raw r = raw_zero();
   if (n_valid <= 0) return r;
+  if constexpr (sizeof(T) == 2) {
+    // a complete bf16 chunk that is only 8- or 4-byte aligned (row strides that are multiples of 4
+    // or 2 elements): two or four loads instead of eight
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+    if (n_valid >= C && (addr & 7) == 0) {
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(p), hi = *reinterpret_cast<const u32x2*>(p + 4);
+      return Raw{lo[0], lo[1], hi[0], hi[1]};
+    }
+    if (n_valid >= C && (addr & 3) == 0) {
+      const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+      return Raw{q[0], q[1], q[2], q[3]};
+    }
+  }
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
     for (int j = 0; j < 4; j++) r[j] = (j < n_valid) ? as_u32(p[j]) : 0u;

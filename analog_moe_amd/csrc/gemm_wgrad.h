@@ -46,10 +46,15 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   const int wn = wave >> 1, wk = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  int b = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int nb = b % p.n_n_blocks; b /= p.n_n_blocks;
-  const int kb = b % p.n_k_blocks;
-  const int e = b / p.n_k_blocks;
+  // Workgroup ids go to the 8 XCDs round-robin.  All tiles of one expert run on one XCD (they
+  // share its rows through that L2) and consecutive experts go to different XCDs, so that a few
+  // heavy experts -- skewed routing -- do not pile up behind one L2 and one eighth of the CUs.
+  const int tiles_per_expert = p.n_k_blocks * p.n_n_blocks;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int e = xcd + 8 * (slot / tiles_per_expert);
+  if (e >= p.E) return;
+  const int tile_id = slot % tiles_per_expert;
+  const int nb = tile_id % p.n_n_blocks, kb = tile_id / p.n_n_blocks;
   const ColBlock kcol = find_col_block(p.bounds, p.n_tiles, kb);
   const int kc0 = kcol.c0, kc1 = kcol.c1;
   const int n0 = nb * kTileCols, n1 = (n0 + kTileCols < p.N) ? n0 + kTileCols : p.N;
