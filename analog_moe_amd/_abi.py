@@ -37,6 +37,7 @@ class BwdWArgs(C.Structure):
         ("offsets", P), ("in_index", P), ("g_index", P), ("ir", P), ("ir_by_expert", C.c_int32),
         ("g_scale", P), ("n_x_rows", C.c_int64), ("n_g_rows", C.c_int64),
         ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
+        ("workspace", P), ("workspace_bytes", C.c_size_t), ("rows_per_chunk", C.c_int32),
     ]
 
 
@@ -66,6 +67,7 @@ PROTOTYPES = {
     "amoe_prepare_sel": (C.c_int, [P, I32, I64, I32, I32, P, P, P, P, P, P, SZ, P]),
     "amoe_offsets_from_sorted": (C.c_int, [P, I64, I32, P, P]),
     "amoe_cvmm_fwd": (C.c_int, [C.POINTER(FwdArgs), P]),
+    "amoe_bwd_w_workspace": (SZ, [C.POINTER(BwdWArgs)]),
     "amoe_cvmm_bwd_w": (C.c_int, [C.POINTER(BwdWArgs), P]),
     "amoe_bwd_x_workspace": (SZ, [I64, I32, I32]),
     "amoe_cvmm_bwd_x": (C.c_int, [C.POINTER(BwdXArgs), P]),

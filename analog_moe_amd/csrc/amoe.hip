@@ -220,6 +220,40 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
 }
 
 // ------------------------------------------------------------------------------ weight gradient
+namespace {
+// Rows per chunk of the weight gradient: enough (expert, chunk, tile) workgroups to fill the chip
+// twice over, chunks of 256 .. 4096 rows; 0 when one chunk per expert already does that.
+struct WgradSplit { int rows_per_chunk; long long slots; int tiles; };
+WgradSplit wgrad_split(const amoe_bwd_w_args* a) {
+  WgradSplit s{0, 0, 0};
+  const int kb = count_col_blocks(a->tile_bounds, a->n_tiles);
+  const int nb = (a->N + kTileCols - 1) / kTileCols;
+  s.tiles = kb * nb;
+  long long R;
+  if (a->rows_per_chunk > 0) {
+    R = ((long long)a->rows_per_chunk + 63) / 64 * 64;
+  } else {
+    const long long target = 4LL * num_compute_units();
+    const long long chunks = (target + s.tiles - 1) / s.tiles;
+    R = chunks > 0 ? (a->M + chunks - 1) / chunks : a->M;
+    R = (R + 255) / 256 * 256;
+    R = R < 256 ? 256 : (R > 4096 ? 4096 : R);
+  }
+  if (R >= a->M) return s;                 // a single chunk everywhere
+  s.rows_per_chunk = (int)R;
+  s.slots = 2LL * a->M / R + 1;            // bound on the chunks of the experts that are cut
+  return s;
+}
+}  // namespace
+
+size_t amoe_bwd_w_workspace(const amoe_bwd_w_args* a) {
+  if (!a || a->M < 1 || a->N < 1 || a->K < 1 || a->E < 1) return 0;
+  if (check_bounds(a->n_tiles, a->tile_bounds, a->K)) return 0;
+  const WgradSplit s = wgrad_split(a);
+  if (s.rows_per_chunk == 0) return 0;
+  return (size_t)s.slots * s.tiles * kWgradTileElems * sizeof(float);
+}
+
 int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
   if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
@@ -247,15 +281,38 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   p.out_stage = aligned(a->grad_w, 16) && (a->N % CH == 0);
   p.buf_ok = a->n_x_rows > 0 && a->n_g_rows > 0 && a->n_x_rows * a->ldx * (long long)es < (1LL << 31) &&
              a->n_g_rows * a->ldg * (long long)es < (1LL << 31);
-  const long long grid = 8LL * ((a->E + 7) / 8) * p.n_k_blocks * p.n_n_blocks;   // see the id mapping in the kernel
-  if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  long long pairs = a->E;                  // (expert, chunk) pairs, worst case
+  if (a->workspace != nullptr && a->M > 0) {
+    const WgradSplit s = wgrad_split(a);
+    if (s.rows_per_chunk > 0) {
+      if (!aligned(a->workspace, 16)) return AMOE_EALIGN;
+      if (a->workspace_bytes < amoe_bwd_w_workspace(a)) return AMOE_EWORKSPACE;
+      if (a->E > kSelMaxExperts) return AMOE_EUNSUPPORTED;
+      p.rows_per_chunk = s.rows_per_chunk;
+      p.partial = static_cast<float*>(a->workspace);
+      pairs = a->M / s.rows_per_chunk + a->E;
+    }
+  }
+  const long long grid = 8LL * ((pairs + 7) / 8) * p.n_k_blocks * p.n_n_blocks;   // see the id mapping in the kernel
+  if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  const long long rgrid = (long long)a->E * p.n_k_blocks * p.n_n_blocks;
   if (a->dtype == AMOE_F32) {
     auto k = &gemm_wgrad_kernel<float>;
     hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
+    if (int rc = launch_rc()) return rc;
+    if (p.rows_per_chunk > 0) {
+      auto r = &wgrad_reduce_kernel<float>;
+      hipLaunchKernelGGL(r, dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
+    }
   } else {
     auto k = &gemm_wgrad_kernel<uint16_t>;
     hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
+    if (int rc = launch_rc()) return rc;
+    if (p.rows_per_chunk > 0) {
+      auto r = &wgrad_reduce_kernel<uint16_t>;
+      hipLaunchKernelGGL(r, dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
+    }
   }
   return launch_rc();
 }

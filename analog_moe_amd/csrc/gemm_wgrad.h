@@ -5,6 +5,10 @@
 // Both operands are staged token-major ("RC": [token][feature], as they lie in memory) and
 // fed to the matrix unit through the transposing LDS read (bf16) or plain reads (fp32); the
 // gradient fragment is the A operand, so a lane holds one kk and runs of 4 consecutive n.
+// With a workspace, an expert with more than two chunks' worth of rows is cut into chunks of
+// rows_per_chunk rows that different workgroups sum (few experts, or a few heavy ones, would
+// otherwise leave most of the chip idle); those workgroups leave fp32 partial tiles, which
+// wgrad_reduce_kernel adds in chunk order in a second launch: no atomics, a fixed summation order.
 // The clip and the optional per-row scale (the gate of the fused layer) are applied to the x
 // operand on its way into LDS; the finished tile leaves through LDS as whole row segments.
 #pragma once
@@ -23,7 +27,16 @@ struct WgradParams {
   int n_k_blocks, n_n_blocks;
   int x_vec, g_vec, out_vec, out_stage;
   int buf_ok;   // x and g small enough for 32-bit byte offsets (buffer loads on interior steps)
+  int rows_per_chunk;            // 0: one workgroup per (expert, tile) walks all rows
+  float* partial;                // [slots][tiles][128*128] fp32 partial tiles of multi-chunk experts
 };
+
+// chunks of an expert with `rows` rows
+__device__ __host__ inline int wgrad_chunks(int rows, int rows_per_chunk) {
+  return (rows_per_chunk > 0 && rows > 2 * rows_per_chunk) ? (rows + rows_per_chunk - 1) / rows_per_chunk : 1;
+}
+
+constexpr int kWgradTileElems = kTileRows * kTileCols;
 
 template <typename T>
 __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradParams p) {
@@ -46,19 +59,74 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   const int wn = wave >> 1, wk = wave & 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  // Workgroup ids go to the 8 XCDs round-robin.  All tiles of one expert run on one XCD (they
-  // share its rows through that L2) and consecutive experts go to different XCDs, so that a few
-  // heavy experts -- skewed routing -- do not pile up behind one L2 and one eighth of the CUs.
+  // Workgroup ids go to the 8 XCDs round-robin.  All tiles of one chunk of rows run on one XCD
+  // (they share those rows through that L2) and consecutive chunks / experts go to different
+  // XCDs, so that a few heavy experts -- skewed routing -- do not pile up behind one L2.
+  // (scratch for the chunk search and the arrival flag lives in the stage buffers, which are idle
+  // then: the two stages fill the LDS budget of two workgroups per CU to the byte)
+  int* const sScanA = reinterpret_cast<int*>(sS);
+  int* const sScanB = sScanA + 4;
+  int* const sFound = sScanA + 8;
   const int tiles_per_expert = p.n_k_blocks * p.n_n_blocks;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int e = xcd + 8 * (slot / tiles_per_expert);
-  if (e >= p.E) return;
+  const int cg = xcd + 8 * (slot / tiles_per_expert);      // index of the (expert, chunk) pair
   const int tile_id = slot % tiles_per_expert;
+  int e = cg, chunk_id = 0, n_chunks = 1, part_slot = 0;
+  if (p.rows_per_chunk > 0) {
+    // chunks per expert -> exclusive prefix; thread tid owns experts [tid*per, (tid+1)*per)
+    const int R = p.rows_per_chunk;
+    const int per = (p.E + kThreads - 1) / kThreads;
+    int mineA = 0, mineB = 0;
+    for (int j = 0; j < per; j++) {
+      const int ee = tid * per + j;
+      if (ee < p.E) {
+        const int rows = p.offsets[ee + 1] - p.offsets[ee];
+        const int c = wgrad_chunks(rows, R);
+        mineA += c;
+        mineB += c > 1 ? c : 0;
+      }
+    }
+    int inclA = mineA, inclB = mineB;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int ua = wave_shfl_up(inclA, d), ub = wave_shfl_up(inclB, d);
+      if (lane >= d) { inclA += ua; inclB += ub; }
+    }
+    if (lane == 63) { sScanA[wave] = inclA; sScanB[wave] = inclB; }
+    if (tid == 0) sFound[0] = -1;
+    __syncthreads();
+    int beforeA = inclA - mineA, beforeB = inclB - mineB;
+    for (int w = 0; w < wave; w++) { beforeA += sScanA[w]; beforeB += sScanB[w]; }
+    for (int j = 0; j < per; j++) {
+      const int ee = tid * per + j;
+      if (ee < p.E) {
+        const int rows = p.offsets[ee + 1] - p.offsets[ee];
+        const int c = wgrad_chunks(rows, R);
+        if (cg >= beforeA && cg < beforeA + c) {
+          sFound[0] = ee; sFound[1] = cg - beforeA; sFound[2] = c; sFound[3] = beforeB;
+        }
+        beforeA += c;
+        beforeB += c > 1 ? c : 0;
+      }
+    }
+    __syncthreads();
+    // (wave-uniform by construction; telling the compiler keeps the tile bookkeeping in scalar registers)
+    e = wave_uniform(sFound[0]); chunk_id = wave_uniform(sFound[1]); n_chunks = wave_uniform(sFound[2]);
+    part_slot = wave_uniform(sFound[3]) + chunk_id;
+    if (e < 0) return;
+    __syncthreads();                       // the scratch is stage memory again from here on
+  } else if (e >= p.E) {
+    return;
+  }
   const int nb = tile_id % p.n_n_blocks, kb = tile_id / p.n_n_blocks;
   const ColBlock kcol = find_col_block(p.bounds, p.n_tiles, kb);
   const int kc0 = kcol.c0, kc1 = kcol.c1;
   const int n0 = nb * kTileCols, n1 = (n0 + kTileCols < p.N) ? n0 + kTileCols : p.N;
-  const int seg0 = p.offsets[e], seg1 = p.offsets[e + 1];
+  int seg0 = p.offsets[e], seg1 = p.offsets[e + 1];
+  if (p.rows_per_chunk > 0 && n_chunks > 1) {
+    seg0 += chunk_id * p.rows_per_chunk;
+    seg1 = seg0 + p.rows_per_chunk < seg1 ? seg0 + p.rows_per_chunk : seg1;
+  }
 
   const T* __restrict__ X = static_cast<const T*>(p.x);
   const T* __restrict__ G = static_cast<const T*>(p.g);
@@ -228,6 +296,22 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
     __syncthreads();
   }
 
+  if (n_chunks > 1) {
+    // leave this chunk's tile in fp32 for wgrad_reduce_kernel
+    float* __restrict__ mine = p.partial + ((int64_t)part_slot * tiles_per_expert + tile_id) * kWgradTileElems;
+#pragma unroll
+    for (int fk = 0; fk < 2; fk++)
+#pragma unroll
+      for (int fn = 0; fn < 2; fn++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          f32x4 v;
+#pragma unroll
+          for (int j = 0; j < 4; j++) v[j] = acc[fn][fk][4 * q + j];
+          *reinterpret_cast<f32x4*>(&mine[(wk * 64 + fk * 32 + l32) * kTileCols + wn * 64 + fn * 32 + 8 * q + 4 * lh]) = v;
+        }
+    return;
+  }
   T* __restrict__ GW = static_cast<T*>(p.grad_w) + (int64_t)e * p.K * p.N;
   if (p.out_stage != 0 && (kc1 - kc0) == kTileCols && (n1 - n0) == kTileCols) {
     // registers -> LDS tile -> whole 256-byte (bf16) / 512-byte (fp32) row segments.  The barrier
@@ -271,6 +355,46 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
         if (nv > 0) store4<T>(GW + (int64_t)kk * p.N + n, v, nv, p.out_vec != 0);
       }
     }
+  }
+}
+
+// Second launch of a row-chunked weight gradient: one workgroup per (expert, tile) adds the fp32
+// partial tiles of a multi-chunk expert in chunk order and writes the tile of grad_w.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(const WgradParams p) {
+  __shared__ int sSum[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tiles = p.n_k_blocks * p.n_n_blocks;
+  const int e = blockIdx.x / tiles, tile_id = blockIdx.x % tiles;
+  const int R = p.rows_per_chunk;
+  const int n_chunks = wgrad_chunks(p.offsets[e + 1] - p.offsets[e], R);
+  if (n_chunks <= 1) return;
+  int before = 0;                          // partial slots of the multi-chunk experts before e
+  for (int ee = tid; ee < e; ee += kThreads) {
+    const int c = wgrad_chunks(p.offsets[ee + 1] - p.offsets[ee], R);
+    before += c > 1 ? c : 0;
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) before += wave_shfl_xor(before, d);
+  if (lane == 0) sSum[wave] = before;
+  __syncthreads();
+  const int slot0 = sSum[0] + sSum[1] + sSum[2] + sSum[3];
+  const int nb = tile_id % p.n_n_blocks, kb = tile_id / p.n_n_blocks;
+  const ColBlock kcol = find_col_block(p.bounds, p.n_tiles, kb);
+  const int n0 = nb * kTileCols;
+  const float* __restrict__ first = p.partial + ((int64_t)slot0 * tiles + tile_id) * kWgradTileElems;
+  T* __restrict__ GW = static_cast<T*>(p.grad_w) + (int64_t)e * p.K * p.N;
+  for (int it = 0; it < kWgradTileElems / (4 * kThreads); it++) {
+    const int idx = (it * kThreads + tid) * 4;
+    const int row = idx / kTileCols, col = idx % kTileCols;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < n_chunks; c++)
+      sum += *reinterpret_cast<const f32x4*>(&first[(int64_t)c * tiles * kWgradTileElems + idx]);
+    const int kk = kcol.c0 + row, n = n0 + col;
+    int nv = kk < kcol.c1 ? p.N - n : 0;
+    nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
+    float v[4] = {sum[0], sum[1], sum[2], sum[3]};
+    if (nv > 0) store4<T>(GW + (int64_t)kk * p.N + n, v, nv, p.out_vec != 0);
   }
 }
 

@@ -48,6 +48,8 @@ __device__ __forceinline__ u32x4 buffer_load_b128(BufRsrc r, uint32_t lane_off, 
   return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0);
 }
 
+// value held by the first active lane, as a scalar
+__device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
 template <typename V>

@@ -113,15 +113,16 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
 def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,
                g_index: Optional[torch.Tensor], *, ir: Optional[torch.Tensor] = None,
                bounds: Optional[Sequence[int]] = None, ir_by_expert: bool = False,
-               g_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """grad_w[e] = sum_i clamp(x[in_index[i]])^T (g_scale[in_index[i]] * g[g_index[i]])."""
+               g_scale: Optional[torch.Tensor] = None, rows_per_chunk: int = 0) -> torch.Tensor:
+    """grad_w[e] = sum_i clamp(x[in_index[i]])^T (g_scale[in_index[i]] * g[g_index[i]]).
+    rows_per_chunk: 0 lets the library decide how the rows of an expert are shared between workgroups."""
     _need_gpu(x, g, offsets, in_index, g_index, ir, g_scale)
     x2, g2 = _rows2d(x), _rows2d(g)
     grad_w = torch.empty((n_experts, x2.shape[1], g2.shape[1]), dtype=x2.dtype, device=x2.device)
     # the library wants the scale per sorted position
     gs = None if g_scale is None else g_scale.detach().reshape(-1).to(x2.dtype)[in_index.long()].contiguous()
     raw.cvmm_bwd_w(get_lib(), _stream(x2), x2, g2, grad_w, offsets, in_index, g_index, _f32c(ir), bounds,
-                   ir_by_expert, gs)
+                   ir_by_expert, gs, rows_per_chunk)
     return grad_w
 
 

@@ -108,7 +108,8 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
 
 
 def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=None,
-               bounds: Optional[Sequence[int]] = None, ir_by_expert: bool = False, g_scale=None):
+               bounds: Optional[Sequence[int]] = None, ir_by_expert: bool = False, g_scale=None,
+               rows_per_chunk: int = 0):
     """x [*, K]; g [*, N]; grad_w [E, K, N] contiguous."""
     _rows(x, "x"); _rows(g, "g")
     if not grad_w.is_contiguous():
@@ -130,6 +131,11 @@ def cvmm_bwd_w(lib, stream, x, g, grad_w, offsets, in_index, g_index=None, ir=No
         raise TypeError("g_scale must be contiguous and share the dtype of x")
     a.g_scale = _p(g_scale)
     a.n_x_rows, a.n_g_rows = x.shape[0], g.shape[0]
+    a.rows_per_chunk = int(rows_per_chunk)
+    need = lib.amoe_bwd_w_workspace(C.byref(a))
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+        a.workspace, a.workspace_bytes = _p(ws), need
     check(lib, lib.amoe_cvmm_bwd_w(C.byref(a), stream), "amoe_cvmm_bwd_w")
 
 

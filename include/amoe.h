@@ -137,8 +137,17 @@ typedef struct amoe_bwd_w_args {
                                             interior path; 0 = unknown: 64-bit addressing) */
   int32_t n_tiles;
   int32_t tile_bounds[AMOE_MAX_TILES + 1];
+  void* workspace;                       /* optional, amoe_bwd_w_workspace(args) bytes: lets several
+                                            workgroups share the rows of one expert (few or heavily
+                                            loaded experts); the sum order stays fixed.  NULL: one
+                                            workgroup per expert and 128x128 tile */
+  size_t workspace_bytes;
+  int32_t rows_per_chunk;                /* 0: the library sizes the row chunks; > 0: rows per chunk
+                                            (rounded up to a multiple of 64) */
 } amoe_bwd_w_args;
 
+/* Bytes of workspace for this call (reads the sizes and tile bounds only). */
+size_t amoe_bwd_w_workspace(const amoe_bwd_w_args* args);
 int amoe_cvmm_bwd_w(const amoe_bwd_w_args* args, void* stream);
 
 /* ---------------------------------------------------------------------------------------

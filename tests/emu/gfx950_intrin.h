@@ -129,6 +129,7 @@ inline uint32_t pack_bf16x2(float lo, float hi) { return emu_f32_to_bf16(lo) | (
 inline float clamp_sym(float x, float r) { return x != x ? -r : (x > r ? r : (x < -r ? -r : x)); }
 inline float fast_sin_rev(float x) { return sinf(6.283185307179586f * x); }
 inline float fast_cos_rev(float x) { return cosf(6.283185307179586f * x); }
+inline int wave_uniform(int v) { return v; }
 inline float fast_log2(float x) { return log2f(x); }
 inline float fast_sqrt(float x) { return sqrtf(x); }
 inline uint32_t umulhi32(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }

@@ -58,6 +58,7 @@ inline float atomicAdd(float* p, float v) {
   while (!r.compare_exchange_weak(old, old + v)) {}
   return old;
 }
+inline void __threadfence() { __atomic_thread_fence(__ATOMIC_SEQ_CST); }
 template <class T> inline T atomicOr(T* p, T v) { return __atomic_fetch_or(p, v, __ATOMIC_RELAXED); }
 template <class T> inline T atomicMax(T* p, T v) {
   T old = __atomic_load_n(p, __ATOMIC_RELAXED);

@@ -167,3 +167,8 @@ def test_argument_errors(emu_ops):
     with pytest.raises(_abi.AmoeError):
         emu_ops.cvmm_fwd(pr["x"], pr["keys"], s_sorted, offsets, in_index, perm, 16, out_bound=12.0)  # no wmax
     assert b"workspace" in lib.amoe_strerror(-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_chunked_weight_gradient(emu_ops, dtype):
+    util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=300)

@@ -135,3 +135,8 @@ def test_companions(ops):
 def test_cpu_tensors_are_rejected(ops):
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.prepare_sel(torch.zeros(4, dtype=torch.int64), 2, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_chunked_weight_gradient(ops, dtype):
+    util.check_row_chunked_wgrad(ops, device="cuda", dtype=dtype, T=4000)

@@ -165,3 +165,28 @@ def adc_steps(pr, ir, lk):
     su = lk["out_bound"] * float(pr["keys"].float().abs().max()) / half * irmax * ntu
     sd = lk["out_bound"] * float(pr["values"].float().abs().max()) / half * irmax * ntd
     return su, sd
+
+
+def check_row_chunked_wgrad(ops, device="cpu", dtype=torch.float32, T=600, D=136, F=72):
+    """The weight gradient with the rows of an expert shared between workgroups (skewed routing: one
+    heavy expert, one empty one) against the oracle, and its run-to-run determinism."""
+    E, k = 5, 2
+    pr = make_problem(21, T, D, E, F, k, dtype=dtype)
+    idx = pr["idx"].clone()
+    idx[idx == 4] = 0                                   # expert 4 empty
+    idx[: T // 2] = torch.tensor([0, 1])                # expert 0 heavy
+    x, g = pr["x"].to(device), torch.randn(T * k, F).to(dtype).to(device)
+    ss, perm, in_index, offsets = ops.prepare_sel(idx.to(device), E, k)
+    ir = torch.full((E, 1), 0.8, device=device)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    want = O.cvmm_bwd_w(np32(x), in_index.cpu().numpy(), ss.cpu().numpy(), np32(g),
+                        np.full((T * k, 1), 0.8, np.float32), E, perm.cpu().numpy(),
+                        dtype="f32" if dtype == torch.float32 else "bf16")
+    outs = []
+    for rows_per_chunk in (64, 64, 192, 1 << 20):
+        got = ops.cvmm_bwd_w(x, g, E, offsets, in_index, perm, ir=ir, ir_by_expert=True,
+                             rows_per_chunk=rows_per_chunk)
+        assert rel_err(np32(got), want) < tol
+        assert float(got[4].abs().max()) == 0.0
+        outs.append(got)
+    assert torch.equal(outs[0], outs[1])
