@@ -27,6 +27,7 @@ class FwdArgs(C.Structure):
         ("wmax", P), ("wmax_cols", C.c_int32),
         ("out_bound", C.c_float), ("out_res", C.c_float),
         ("relu", C.c_int32), ("range_flag", P),
+        ("xq_out", P), ("ldxq", C.c_int64), ("xq_ir", P), ("xq_inp_res", C.c_float), ("x_is_quantized", C.c_int32),
     ]
 
 

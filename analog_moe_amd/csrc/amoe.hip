@@ -58,6 +58,7 @@ inline int persistent_grid(int row_tiles, int col_blocks) {
 // Every tile of the launch is interior: the FAST instantiation applies.
 inline bool rows_all_interior(const RowsParams& p, int mode, int bk) {
   if (!p.a_vec || !p.w_vec || !p.out_stage || !p.buf_ok || p.abs_max != nullptr) return false;
+  if (p.xq_out != nullptr && !p.xq_stage) return false;
   // forward: the edge-free code has the clip-and-quantise input stage or none at all
   if (mode != MODE_BWDX && (p.ir != nullptr) != (p.inp_res > 0.f)) return false;
   if (p.noise != nullptr && !p.noise_vec) return false;
@@ -112,7 +113,7 @@ const char* amoe_strerror(int rc) {
 // ------------------------------------------------------------------------------ selection
 size_t amoe_prepare_sel_workspace(int64_t M, int32_t E) {
   if (M < 0 || E < 1) return 0;
-  const int64_t units = (M + kSelUnit - 1) / kSelUnit;
+  const int64_t units = (M + sel_unit(M) - 1) / sel_unit(M);
   return (size_t)(units > 0 ? units : 1) * (size_t)E * sizeof(int32_t);
 }
 
@@ -128,7 +129,8 @@ int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, 
   if (workspace_bytes < amoe_prepare_sel_workspace(M, E)) return AMOE_EWORKSPACE;
   SelParams p;
   p.sel = sel; p.sel_is_i64 = sel_is_i64; p.M = M; p.E = E; p.k = k;
-  p.n_units = (int)((M + kSelUnit - 1) / kSelUnit);
+  p.unit = sel_unit(M);
+  p.n_units = (int)((M + p.unit - 1) / p.unit);
   p.key_bits = 0;
   while ((1 << p.key_bits) < E) p.key_bits++;
   p.sel_sorted = sel_sorted; p.perm = perm; p.in_index = in_index; p.offsets = offsets;
@@ -175,10 +177,14 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   if ((gen_noise || adc) && (!a->wmax || (a->wmax_cols != 1 && a->wmax_cols != a->N))) return AMOE_ESHAPE;
   if (gen_noise && (a->N % 2)) return AMOE_EUNSUPPORTED;
   if (a->noise && (a->ldnoise < a->N)) return AMOE_ESHAPE;
+  if (a->xq_out && (!a->xq_ir || !(a->xq_inp_res > 0.f))) return AMOE_EINVAL;
+  if (a->xq_out && a->ldxq < a->N) return AMOE_ESHAPE;
+  if (a->x_is_quantized && (!a->ir || !(a->inp_res > 0.f) || a->abs_max || a->n_tiles != 1)) return AMOE_EINVAL;
   const size_t es = esize(a->dtype);
   if (!aligned(a->x, es) || !aligned(a->w, es) || !aligned(a->out, es) || !aligned(a->offsets, 4) ||
       !aligned(a->in_index, 4) || !aligned(a->out_index, 4) || !aligned(a->ir, 4) || !aligned(a->abs_max, 4) ||
-      !aligned(a->noise, 4) || !aligned(a->wmax, 4) || !aligned(a->range_flag, 4) || !aligned(a->noise_seed_dev, 8))
+      !aligned(a->noise, 4) || !aligned(a->wmax, 4) || !aligned(a->range_flag, 4) || !aligned(a->noise_seed_dev, 8) ||
+      !aligned(a->xq_out, es) || !aligned(a->xq_ir, 4))
     return AMOE_EALIGN;
 
   const int CH = a->dtype == AMOE_F32 ? 4 : 8;
@@ -200,6 +206,10 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   p.out_bound = a->out_bound;
   p.out_half_states = (adc && a->out_res > 0.f) ? 0.5f * fmaxf(a->out_res, 1.0f / a->out_res) : 0.f;
   p.relu = a->relu; p.range_flag = a->range_flag;
+  p.xq_out = a->xq_out; p.ldxq = a->ldxq; p.xq_ir = a->xq_ir; p.xq_inp_res = a->xq_inp_res;
+  p.xq_vec = a->xq_out && aligned(a->xq_out, 16) && (a->ldxq % 4 == 0);
+  p.xq_stage = a->xq_out && aligned(a->xq_out, 16) && (a->ldxq % CH == 0);
+  p.a_prequant = a->x_is_quantized;
   const bool w_kc = a->w_stride_n != 1;
   p.a_vec = aligned(a->x, 16) && (a->ldx % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   p.w_vec = aligned(a->w, 16) && (a->w_stride_e % CH == 0) &&

@@ -35,6 +35,8 @@ struct RowsParams {
   const float* noise; int64_t noise_ts, ldnoise; float noise_std; uint64_t seed; const uint64_t* seed_dev;
   const float* wmax; int wmax_cols; float out_bound, out_half_states; int relu;
   int32_t* range_flag;
+  void* xq_out; int64_t ldxq; const float* xq_ir; float xq_inp_res; int xq_stage, xq_vec;  // DAC image of the result
+  int a_prequant;                    // the gathered operand already is such an image: no input stage
   // input gradient
   const void* xf; int64_t ldxf; const int32_t* xf_index; const void* gate;
   float* irg_partial; int32_t* notclip_count; int relu_mask;
@@ -150,8 +152,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const bool has_ir = FWD && p.ir != nullptr;
   const bool has_amax = !FAST && FWD && p.abs_max != nullptr;
   const bool quant = FWD && p.inp_res > 0.f;
-  const bool dac = has_ir || has_amax || quant;
-  const bool dac_ir_quant = has_ir && quant && !has_amax;   // the common analog case: tight code
+  const bool prequant = FWD && p.a_prequant != 0;          // the caller did the input stage already
+  const bool dac = (has_ir || has_amax || quant) && !prequant;
+  const bool dac_ir_quant = has_ir && quant && !has_amax && !prequant;   // the common analog case: tight code
   const bool codes_mode = IS_BF16 && quant;   // feed integer codes, scale the accumulator
   const bool adc_clip = FWD && p.out_bound > 0.f;
   const bool adc_quant = adc_clip && p.out_half_states > 0.f;
@@ -580,7 +583,26 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       }
     }
 
-    const bool staged = FAST || (p.out_stage != 0 && (c1 - c0) == kTileCols);
+    // The tile leaves once as the result and, when the caller wants it (forward), a second time as
+    // the DAC image of the result for the projection that follows: clamp / scale / round of the
+    // value as stored in T, so that projection's input stage has nothing left to do.
+    const float q_r = (FWD && p.xq_out != nullptr) ? p.xq_ir[e] : 1.f;
+    const float q_rinv = 1.0f / q_r, q_res = p.xq_inp_res, q_resinv = 1.0f / p.xq_inp_res;
+    auto as_codes = [&](float (&v)[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float x = v[j];
+        if constexpr (IS_BF16) x = as_f32((uint32_t)Elem<T>::cvt(x) << 16);
+        x = clamp_sym(x, q_r);
+        const float c = rintf(div_by(div_by(x, q_r, q_rinv), q_res, q_resinv));
+        v[j] = IS_BF16 ? c : c * q_res;
+      }
+    };
+    const int n_out = (FWD && p.xq_out != nullptr) ? 2 : 1;
+    for (int pass = 0; pass < n_out; pass++) {
+    T* __restrict__ DST = pass == 0 ? OUT : static_cast<T*>(p.xq_out);
+    const int64_t ldd = pass == 0 ? p.ldo : p.ldxq;
+    const bool staged = FAST || ((pass == 0 ? p.out_stage : p.xq_stage) != 0 && (c1 - c0) == kTileCols);
     if (staged) {
       // registers -> LDS tile -> whole 256-byte (bf16) row segments to global memory
       // (the input gradient may still be reading the parked mask tile from the other stage)
@@ -598,6 +620,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
                 float v[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
+                if (pass == 1) as_codes(v);
                 store4<T>(&sOut[rl * LDO + wc * 64 + fi * 32 + 8 * q + 4 * lh], v, 4, true);
               }
           }
@@ -610,7 +633,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           const int rl = tid / OCPR + ORPP * i;
           const int orow = sOrow[h * OUT_ROWS + rl];
           if (orow >= 0)
-            *reinterpret_cast<Raw*>(OUT + (int64_t)orow * p.ldo + c0 + (tid % OCPR) * CH) =
+            *reinterpret_cast<Raw*>(DST + (int64_t)orow * ldd + c0 + (tid % OCPR) * CH) =
                 *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
         }
         __syncthreads();
@@ -630,10 +653,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             float v[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
-            if (nv > 0) store4<T>(OUT + (int64_t)orow * p.ldo + col, v, nv, p.out_vec != 0);
+            if (pass == 1) as_codes(v);
+            if (nv > 0) store4<T>(DST + (int64_t)orow * ldd + col, v, nv, (pass == 0 ? p.out_vec : p.xq_vec) != 0);
           }
       }
       __syncthreads();
+    }
     }
     if (use_ir_bw) {     // sRed was written before the barriers above
       if (tid < kTileRows && row0 + tid < row_end)

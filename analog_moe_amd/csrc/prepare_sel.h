@@ -11,12 +11,18 @@
 
 namespace amoe {
 
-constexpr int kSelUnit = 1024;      // elements per wave
+constexpr int kSelUnitMax = 1024;   // elements per wave: 64 .. 1024, fewer for short inputs so that
+                                    // the sort still spreads over the chip (see sel_unit)
+__host__ __device__ inline int sel_unit(long long M) {
+  int u = 64;
+  while (u < kSelUnitMax && M / u > 2048) u <<= 1;   // aim at <= 2048 units
+  return u < 256 ? 256 : u;
+}
 constexpr int kSelMaxExperts = 2048;
 
 struct SelParams {
   const void* sel; int sel_is_i64;
-  long long M; int E, k, n_units, key_bits;
+  long long M; int E, k, n_units, key_bits, unit;
   int32_t* sel_sorted; int32_t* perm; int32_t* in_index; int32_t* offsets; int32_t* bad_flag;
   int32_t* unit_hist;               // workspace [n_units][E]
 };
@@ -38,8 +44,8 @@ __global__ __launch_bounds__(kThreads) void sel_hist_kernel(const SelParams p) {
   const int unit = blockIdx.x * 4 + wave;
   bool any_bad = false;
   if (unit < p.n_units) {
-    for (int it = 0; it < kSelUnit / 64; it++) {
-      const long long i = (long long)unit * kSelUnit + it * 64 + lane;
+    for (int it = 0; it < p.unit / 64; it++) {
+      const long long i = (long long)unit * p.unit + it * 64 + lane;
       if (i < p.M) {
         bool bad;
         const int key = sel_key(p, i, bad);
@@ -122,8 +128,8 @@ __global__ __launch_bounds__(kThreads) void sel_scatter_kernel(const SelParams p
   const int unit = blockIdx.x * 4 + wave;
   int* my_base = &base[wave * p.E];
   const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
-  for (int it = 0; it < kSelUnit / 64; it++) {
-    const long long i = (long long)unit * kSelUnit + it * 64 + lane;
+  for (int it = 0; it < p.unit / 64; it++) {
+    const long long i = (long long)unit * p.unit + it * 64 + lane;
     const bool valid = unit < p.n_units && i < p.M;
     bool bad;
     const int key = valid ? sel_key(p, i, bad) : 0;

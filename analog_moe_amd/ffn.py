@@ -59,12 +59,17 @@ class AnalogMoEFFN(torch.autograd.Function):
             wd = ops.weight_abs_max(values, cfg.noise_per_channel)
         common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
                       noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
+        # the up-projection also emits the down-projection's DAC image of its result (each row belongs
+        # to one expert, so the image is made once instead of once per block of output columns)
+        chain = ir_dn is not None and cfg.inp_res > 0 and ntd == 1
         p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, bounds=cfg.bounds_up,
                           noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True,
-                          noise_seed_dev=cfg.noise_seed_dev, **common)
-        z = ops.cvmm_fwd(p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn, bounds=cfg.bounds_down,
-                         noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
-                         noise_seed_dev=cfg.noise_seed_dev, **common)
+                          noise_seed_dev=cfg.noise_seed_dev, xq_ir=ir_dn[:, 0].contiguous() if chain else None,
+                          xq_inp_res=cfg.inp_res, **common)
+        p1, p1q = p1 if chain else (p1, None)
+        z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn,
+                         bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
+                         noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
         y = ops.gate_reduce(z, gate)
         ctx.save_for_backward(x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn)
         ctx.cfg = cfg

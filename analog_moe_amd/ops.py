@@ -95,19 +95,23 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
              bounds: Optional[Sequence[int]] = None, noise: Optional[torch.Tensor] = None,
              noise_std: float = 0.0, noise_seed: int = 0, wmax: Optional[torch.Tensor] = None,
              out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
-             ir_by_expert: bool = False, noise_seed_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+             ir_by_expert: bool = False, noise_seed_dev: Optional[torch.Tensor] = None,
+             xq_ir: Optional[torch.Tensor] = None, xq_inp_res: float = -1.0, x_is_quantized: bool = False):
     """out[out_index[i]] = analog(x[in_index[i]]) @ w[sel_sorted[i]] -> [n_out_rows, N].
     ir: [M, n_tiles] per sorted position, or the [E, n_tiles] table with ir_by_expert.
-    noise_seed_dev: optional int64 device word added to noise_seed by the kernel."""
+    noise_seed_dev: optional int64 device word added to noise_seed by the kernel.
+    xq_ir ([E] fp32) + xq_inp_res: also return the input-stage image of the result for the projection
+    that follows (-> (out, xq)); x_is_quantized: x is such an image made for this call."""
     _need_gpu(x, w, sel_sorted, offsets, in_index, out_index, ir, abs_max, noise, wmax)
     x2 = _rows2d(x)
     if w.stride(2) != 1 and w.stride(1) != 1:
         w = w.contiguous()
     out = torch.empty((n_out_rows, w.shape[2]), dtype=x2.dtype, device=x2.device)
+    xq = torch.empty_like(out) if xq_ir is not None else None
     raw.cvmm_fwd(get_lib(), _stream(x2), x2, w, out, sel_sorted, offsets, in_index, out_index, _f32c(ir),
                  _f32c(abs_max), inp_res, bounds, _f32c(noise), noise_std, noise_seed, _f32c(wmax), out_bound,
-                 out_res, relu, None, ir_by_expert, noise_seed_dev)
-    return out
+                 out_res, relu, None, ir_by_expert, noise_seed_dev, xq, _f32c(xq_ir), xq_inp_res, x_is_quantized)
+    return out if xq is None else (out, xq)
 
 
 def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,

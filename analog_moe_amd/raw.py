@@ -66,7 +66,8 @@ def offsets_from_sorted(lib, stream, sel_sorted, E: int, offsets):
 def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=None, ir=None, abs_max=None,
              inp_res: float = -1.0, bounds: Optional[Sequence[int]] = None, noise=None, noise_std: float = 0.0,
              noise_seed: int = 0, wmax=None, out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
-             range_flag=None, ir_by_expert: bool = False, noise_seed_dev=None):
+             range_flag=None, ir_by_expert: bool = False, noise_seed_dev=None, xq_out=None, xq_ir=None,
+             xq_inp_res: float = -1.0, x_is_quantized: bool = False):
     """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N]."""
     _rows(x, "x"); _rows(out, "out")
     a = FwdArgs()
@@ -104,6 +105,12 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
         a.wmax, a.wmax_cols = _p(wmax), wmax.numel() // E
     a.out_bound, a.out_res = float(out_bound), float(out_res)
     a.relu, a.range_flag = int(bool(relu)), _p(range_flag)
+    if xq_out is not None:
+        _rows(xq_out, "xq_out")
+        if xq_out.dtype != x.dtype or xq_out.shape != out.shape:
+            raise ValueError("xq_out must match out")
+        a.xq_out, a.ldxq, a.xq_ir, a.xq_inp_res = _p(xq_out), xq_out.stride(0), _p(_f32(xq_ir, "xq_ir")), float(xq_inp_res)
+    a.x_is_quantized = int(bool(x_is_quantized))
     check(lib, lib.amoe_cvmm_fwd(C.byref(a), stream), "amoe_cvmm_fwd")
 
 

@@ -107,6 +107,17 @@ typedef struct amoe_fwd_args {
   int32_t relu;                  /* fuse max(., 0) into the store */
   int32_t* range_flag;           /* device int32 or NULL: set to 1 if |a| > 1 is met before
                                     quantising (cvmm.py:162 asserts this) */
+  /* Chaining two projections (no counterpart in the reference, which re-runs the input stage of
+     the second projection for every block of its output columns): */
+  void* xq_out;                  /* optional second output [n_out_rows, N], dtype: the input stage
+                                    (clamp to +-xq_ir[e], / xq_ir[e], round to xq_inp_res) of the
+                                    projection that consumes `out`, applied to `out` as stored.
+                                    bf16 holds the integer codes, fp32 codes * xq_inp_res */
+  int64_t ldxq;
+  const float* xq_ir;            /* [E] input range of that projection (it must have one K-tile) */
+  float xq_inp_res;              /* its quantisation step, > 0 */
+  int32_t x_is_quantized;        /* != 0: x is such an image made with this call's ir / inp_res:
+                                    the input stage is skipped, the rescale is not */
 } amoe_fwd_args;
 
 int amoe_cvmm_fwd(const amoe_fwd_args* args, void* stream);

@@ -172,3 +172,8 @@ def test_argument_errors(emu_ops):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_row_chunked_weight_gradient(emu_ops, dtype):
     util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=300)
+
+
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
+def test_chained_projections(emu_ops, dtype, D, F):
+    util.check_chained_projections(emu_ops, dtype=dtype, T=60, D=D, F=F)

@@ -140,3 +140,9 @@ def test_cpu_tensors_are_rejected(ops):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_row_chunked_weight_gradient(ops, dtype):
     util.check_row_chunked_wgrad(ops, device="cuda", dtype=dtype, T=4000)
+
+
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 256, 128), (torch.bfloat16, 256, 128), (torch.bfloat16, 72, 40),
+                                       (torch.float32, 100, 36)])
+def test_chained_projections(ops, dtype, D, F):
+    util.check_chained_projections(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)

@@ -190,3 +190,28 @@ def check_row_chunked_wgrad(ops, device="cpu", dtype=torch.float32, T=600, D=136
         assert float(got[4].abs().max()) == 0.0
         outs.append(got)
     assert torch.equal(outs[0], outs[1])
+
+
+def check_chained_projections(ops, device="cpu", dtype=torch.float32, T=100, D=128, F=128, E=3, k=2):
+    """The DAC image that the up-projection emits for the down-projection gives bit-identical
+    down-projection results to running the down-projection's own input stage."""
+    pr = make_problem(17, T, D, E, F, k, dtype=dtype)
+    pr = {n: t.to(device) for n, t in pr.items()}
+    ss, perm, in_index, offsets = ops.prepare_sel(pr["idx"], E, k)
+    M = T * k
+    ir_up = torch.linspace(0.9, 1.6, E, device=device).reshape(E, 1)
+    ir_dn = torch.linspace(0.5, 1.1, E, device=device).reshape(E, 1)
+    res = 1 / 127
+    p1, p1q = ops.cvmm_fwd(pr["x"], pr["keys"], ss, offsets, in_index, perm, M, ir=ir_up, ir_by_expert=True,
+                           inp_res=res, relu=True, xq_ir=ir_dn[:, 0].contiguous(), xq_inp_res=res)
+    p1_alone = ops.cvmm_fwd(pr["x"], pr["keys"], ss, offsets, in_index, perm, M, ir=ir_up, ir_by_expert=True,
+                            inp_res=res, relu=True)
+    assert torch.equal(p1, p1_alone)
+    # rows of p1 are flat (token, head) positions: row i belongs to expert idx.flat[i]
+    ir_rows = ir_dn.cpu().numpy()[pr["idx"].reshape(-1).cpu().numpy()]
+    want_a, want_codes = O.dac(np32(p1), ir_rows, None, res)
+    np.testing.assert_array_equal(np32(p1q), want_a if dtype == torch.float32 else want_codes)
+    z_chain = ops.cvmm_fwd(p1q, pr["values"], ss, offsets, perm, None, M, ir=ir_dn, ir_by_expert=True,
+                           inp_res=res, x_is_quantized=True)
+    z_plain = ops.cvmm_fwd(p1, pr["values"], ss, offsets, perm, None, M, ir=ir_dn, ir_by_expert=True, inp_res=res)
+    assert torch.equal(z_chain, z_plain)
