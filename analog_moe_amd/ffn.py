@@ -35,6 +35,17 @@ class FFNConfig:
     noise_down: Optional[torch.Tensor] = None
 
 
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority), for the bandwidth-bound companions."""
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
+
+
 class AnalogMoEFFN(torch.autograd.Function):
     """y[t] = sum_j gate[t,j] * A(relu(A(x[t], keys[e_tj])), values[e_tj]).
     input_range: [2, E, n_tiles] (row 0 up-, row 1 down-projection) or None."""
@@ -89,11 +100,18 @@ class AnalogMoEFFN(torch.autograd.Function):
         irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
                     input_min_percentage=cfg.input_min_percentage)
         tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+        # the gate gradient only streams z and dy through HBM; it runs on a second stream next to the
+        # weight gradient, whose workgroups leave registers and wave slots free on every CU
+        main, side = torch.cuda.current_stream(), _side_stream(x.device)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+        grad_gate.record_stream(main)
         grad_values = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, bounds=cfg.bounds_down, g_scale=gate,
                                      **by)
         gp1, irg_dn = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate, ir=ir_dn,
                                      bounds=cfg.bounds_down, relu_mask=True, **irkw, **by)
-        grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+        main.wait_stream(side)
         grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
         full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
                                       bounds=cfg.bounds_up, **irkw, **by)
