@@ -33,7 +33,7 @@ def emu_ops():
     ops._LIB, ops._stream, ops._need_gpu = saved
 
 
-@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (66, 4, 2), (1500, 8, 2), (5000, 130, 4), (70000, 515, 3)])
+@pytest.mark.parametrize("M,E,k", [(0, 4, 1), (1, 1, 1), (66, 4, 2), (1500, 8, 2), (5000, 130, 4), (20000, 300, 3)])
 def test_prepare_sel_bit_exact(emu_ops, M, E, k):
     M -= M % k
     sel = torch.from_numpy(np.random.default_rng(M).integers(0, E, size=M))
@@ -171,7 +171,7 @@ def test_argument_errors(emu_ops):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_row_chunked_weight_gradient(emu_ops, dtype):
-    util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=300)
+    util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=200)
 
 
 @pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
