@@ -55,7 +55,7 @@ class BwdXArgs(C.Structure):
         ("gradient_relative", C.c_int32), ("gradient_scale", C.c_float),
         ("decay", C.c_float), ("input_min_percentage", C.c_float),
         ("relu_mask", C.c_int32),
-        ("workspace", P), ("workspace_bytes", C.c_size_t),
+        ("workspace", P), ("workspace_bytes", C.c_size_t), ("xc_out", P), ("ldxc", C.c_int64),
     ]
 
 

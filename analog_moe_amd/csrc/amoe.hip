@@ -59,6 +59,7 @@ inline int persistent_grid(int row_tiles, int col_blocks) {
 inline bool rows_all_interior(const RowsParams& p, int mode, int bk) {
   if (!p.a_vec || !p.w_vec || !p.out_stage || !p.buf_ok || p.abs_max != nullptr) return false;
   if (p.xq_out != nullptr && !p.xq_stage) return false;
+  if (p.xc_out != nullptr && !p.xc_vec) return false;
   // forward: the edge-free code has the clip-and-quantise input stage or none at all
   if (mode != MODE_BWDX && (p.ir != nullptr) != (p.inp_res > 0.f)) return false;
   if (p.noise != nullptr && !p.noise_vec) return false;
@@ -346,6 +347,8 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   const bool use_ir = a->ir != nullptr;
   if ((use_ir || a->relu_mask) && (!a->x || !a->xf_index)) return AMOE_ENULL;
   if (use_ir && (!a->ir_grad || !a->workspace)) return AMOE_ENULL;
+  if (a->xc_out && (!a->x || !a->xf_index)) return AMOE_ENULL;
+  if (a->xc_out && a->ldxc < a->K) return AMOE_ESHAPE;
   if (a->ldg < a->N || a->ldo < a->K || (a->x && a->ldx < a->K) || a->w_stride_k < a->N) return AMOE_ESHAPE;
   const size_t es = esize(a->dtype);
   if (!aligned(a->g, es) || !aligned(a->w, es) || !aligned(a->grad_x_full, es) || !aligned(a->x, es) ||
@@ -365,6 +368,8 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles);
   p.ir = a->ir; p.ir_cols = a->n_tiles; p.ir_by_expert = a->ir_by_expert; p.inp_res = -1.f;
   p.xf = a->x; p.ldxf = a->ldx; p.xf_index = a->xf_index; p.gate = a->gate; p.relu_mask = a->relu_mask;
+  p.xc_out = a->xc_out; p.ldxc = a->ldxc;
+  p.xc_vec = a->xc_out && aligned(a->xc_out, 16) && (a->ldxc % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (use_ir) {
     const size_t need = (size_t)p.n_col_blocks * a->M * sizeof(float) + (size_t)grid * sizeof(int32_t);

@@ -40,6 +40,7 @@ struct RowsParams {
   // input gradient
   const void* xf; int64_t ldxf; const int32_t* xf_index; const void* gate;
   float* irg_partial; int32_t* notclip_count; int relu_mask;
+  void* xc_out; int64_t ldxc; int xc_vec;   // gate * clamp(x): the weight gradient's x operand, made once here
   // vector-access permissions (alignment checked on the host)
   int a_vec, w_vec, out_vec, out_stage, noise_vec, xf_vec;   // out_stage: 16-byte row segments
   int buf_ok;   // operands small enough for 32-bit byte offsets (buffer loads in the interior path)
@@ -558,6 +559,17 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             } else if (XF != nullptr && nv > 0) {
               load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, FAST || p.xf_vec != 0);
             }
+            if (p.xc_out != nullptr) {      // the clipped, gate-scaled input for the weight gradient
+              float pc[4];
+#pragma unroll
+              for (int j = 0; j < 4; j++) pc[j] = (use_ir_bw ? clamp_sym(xv[j], ir_r) : xv[j]) * gate_r;
+              if (xf_stage) {               // in place: it leaves with the tile below
+                const int nst = (p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK;
+                store4<T>(&sStage[(nst & 1) * STAGE + rl * LDO + col - c0], pc, 4, true);
+              } else if (nv > 0) {
+                store4<T>(static_cast<T*>(p.xc_out) + (int64_t)xrow * p.ldxc + col, pc, nv, p.xc_vec != 0);
+              }
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
               float g = acc[fi][ti][4 * q + j];
@@ -635,6 +647,16 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           if (orow >= 0)
             *reinterpret_cast<Raw*>(DST + (int64_t)orow * ldd + c0 + (tid % OCPR) * CH) =
                 *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+        }
+        if (xf_stage && p.xc_out != nullptr) {     // the parked input tile, clipped and scaled in place
+          const T* __restrict__ sXF = sStage + (sOut == sStage ? STAGE : 0);
+#pragma unroll
+          for (int i = 0; i < OUT_ROWS / ORPP; i++) {
+            const int rl = tid / OCPR + ORPP * i;
+            if (row0 + rl < row_end)
+              *reinterpret_cast<Raw*>(static_cast<T*>(p.xc_out) + (int64_t)sXrow[rl] * p.ldxc + c0 + (tid % OCPR) * CH) =
+                  *reinterpret_cast<const Raw*>(&sXF[rl * LDO + (tid % OCPR) * CH]);
+          }
         }
         __syncthreads();
       }

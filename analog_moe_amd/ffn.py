@@ -100,6 +100,11 @@ class AnalogMoEFFN(torch.autograd.Function):
         irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
                     input_min_percentage=cfg.input_min_percentage)
         tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+        # the input gradient reads p1 for its masks anyway; it also leaves gate * clamp(p1), which is the
+        # x operand of the weight gradient (otherwise every block of its output columns clips and scales)
+        gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
+                                          ir=ir_dn, bounds=cfg.bounds_down, relu_mask=True, want_xc=True,
+                                          **irkw, **by)
         # the gate gradient only streams z and dy through HBM; it runs on a second stream next to the
         # weight gradient, whose workgroups leave registers and wave slots free on every CU
         main, side = torch.cuda.current_stream(), _side_stream(x.device)
@@ -107,12 +112,9 @@ class AnalogMoEFFN(torch.autograd.Function):
         with torch.cuda.stream(side):
             grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
         grad_gate.record_stream(main)
-        grad_values = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, bounds=cfg.bounds_down, g_scale=gate,
-                                     **by)
-        gp1, irg_dn = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate, ir=ir_dn,
-                                     bounds=cfg.bounds_down, relu_mask=True, **irkw, **by)
-        main.wait_stream(side)
+        grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
         grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
+        main.wait_stream(side)
         full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
                                       bounds=cfg.bounds_up, **irkw, **by)
         grad_x = ops.ksum(full, k) if k > 1 else full

@@ -135,8 +135,10 @@ def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index:
                xf_index: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
                ir: Optional[torch.Tensor] = None, bounds: Optional[Sequence[int]] = None,
                gradient_relative: bool = True, gradient_scale: float = 1.0, decay: float = 0.0,
-               input_min_percentage: float = 0.95, relu_mask: bool = False, ir_by_expert: bool = False):
-    """Returns (grad_x_full [n_out_rows, K], ir_grad [M, n_tiles] or None)."""
+               input_min_percentage: float = 0.95, relu_mask: bool = False, ir_by_expert: bool = False,
+               want_xc: bool = False):
+    """Returns (grad_x_full [n_out_rows, K], ir_grad [M, n_tiles] or None) and, with want_xc, also
+    gate * clamp(x, +-ir) in the layout of x: the x operand of the weight gradient of the same projection."""
     _need_gpu(g, w, offsets, g_index, out_index, x, xf_index, gate, ir)
     lib = get_lib()
     g2 = _rows2d(g)
@@ -153,10 +155,11 @@ def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index:
         ir_grad = torch.empty((M, n_tiles), dtype=torch.float32, device=g2.device)
         ws = torch.empty(max(raw.bwd_x_workspace_bytes(lib, M, K, n_tiles), 4), dtype=torch.uint8, device=g2.device)
     gate_c = None if gate is None else gate.detach().reshape(-1).to(g2.dtype).contiguous()
+    xc = torch.empty_like(x2) if (want_xc and x2 is not None) else None
     raw.cvmm_bwd_x(lib, _stream(g2), g2, w, full, offsets, g_index, out_index, x2, xf_index, gate_c, ir32, ir_grad,
                    bounds, gradient_relative, gradient_scale, decay, input_min_percentage, relu_mask, ws,
-                   ir_by_expert)
-    return full, ir_grad
+                   ir_by_expert, xc)
+    return (full, ir_grad, xc) if want_xc else (full, ir_grad)
 
 
 # ------------------------------------------------------------------------------ companions

@@ -153,7 +153,7 @@ def bwd_x_workspace_bytes(lib, M: int, K: int, n_tiles: int) -> int:
 def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=None, xf_index=None, gate=None,
                ir=None, ir_grad=None, bounds: Optional[Sequence[int]] = None, gradient_relative: bool = True,
                gradient_scale: float = 1.0, decay: float = 0.0, input_min_percentage: float = 0.95,
-               relu_mask: bool = False, workspace=None, ir_by_expert: bool = False):
+               relu_mask: bool = False, workspace=None, ir_by_expert: bool = False, xc_out=None):
     """g [*, N]; w [E, K, N] with N contiguous; grad_x_full [R_out, K]; x [*, K] forward input."""
     _rows(g, "g"); _rows(grad_x_full, "grad_x_full")
     a = BwdXArgs()
@@ -183,6 +183,11 @@ def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=No
     a.relu_mask = int(bool(relu_mask))
     if workspace is not None:
         a.workspace, a.workspace_bytes = _p(workspace), workspace.numel() * workspace.element_size()
+    if xc_out is not None:
+        _rows(xc_out, "xc_out")
+        if x is None or xc_out.dtype != x.dtype or xc_out.shape != x.shape:
+            raise ValueError("xc_out must match x")
+        a.xc_out, a.ldxc = _p(xc_out), xc_out.stride(0)
     check(lib, lib.amoe_cvmm_bwd_x(C.byref(a), stream), "amoe_cvmm_bwd_x")
 
 

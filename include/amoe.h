@@ -195,6 +195,13 @@ typedef struct amoe_bwd_x_args {
   float decay;  float input_min_percentage;
   int32_t relu_mask;
   void* workspace;  size_t workspace_bytes;
+  void* xc_out;                          /* optional [rows of x, K], dtype: gate * clamp(x, +-ir) at row
+                                            xf_index[i] -- the x operand of the weight gradient of
+                                            the same projection (amoe_cvmm_bwd_w then runs without
+                                            ir and g_scale).  No counterpart in the reference, which
+                                            clips inside its weight-gradient kernel for every block
+                                            of output columns.  Needs x */
+  int64_t ldxc;
 } amoe_bwd_x_args;
 
 size_t amoe_bwd_x_workspace(int64_t M, int32_t K, int32_t n_tiles);

@@ -177,3 +177,8 @@ def test_row_chunked_weight_gradient(emu_ops, dtype):
 @pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
 def test_chained_projections(emu_ops, dtype, D, F):
     util.check_chained_projections(emu_ops, dtype=dtype, T=60, D=D, F=F)
+
+
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
+def test_clipped_input_for_the_weight_gradient(emu_ops, dtype, D, F):
+    util.check_clipped_input_output(emu_ops, dtype=dtype, T=60, D=D, F=F)

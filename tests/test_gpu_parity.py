@@ -146,3 +146,9 @@ def test_row_chunked_weight_gradient(ops, dtype):
                                        (torch.float32, 100, 36)])
 def test_chained_projections(ops, dtype, D, F):
     util.check_chained_projections(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)
+
+
+@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 256, 128), (torch.bfloat16, 256, 128), (torch.bfloat16, 256, 192),
+                                       (torch.bfloat16, 72, 40)])
+def test_clipped_input_for_the_weight_gradient(ops, dtype, D, F):
+    util.check_clipped_input_output(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)

@@ -215,3 +215,27 @@ def check_chained_projections(ops, device="cpu", dtype=torch.float32, T=100, D=1
                            inp_res=res, x_is_quantized=True)
     z_plain = ops.cvmm_fwd(p1, pr["values"], ss, offsets, perm, None, M, ir=ir_dn, ir_by_expert=True, inp_res=res)
     assert torch.equal(z_chain, z_plain)
+
+
+def check_clipped_input_output(ops, device="cpu", dtype=torch.float32, T=100, D=128, F=128, E=3, k=2):
+    """gate * clamp(x) left by the input gradient feeds the weight gradient: same weight gradient, bit
+    for bit, as clipping and scaling inside the weight-gradient kernel."""
+    pr = make_problem(19, T, D, E, F, k, dtype=dtype)
+    pr = {n: t.to(device) for n, t in pr.items()}
+    ss, perm, in_index, offsets = ops.prepare_sel(pr["idx"], E, k)
+    M = T * k
+    p1 = torch.randn(M, F).to(dtype).to(device)
+    ir_dn = torch.linspace(0.5, 1.1, E, device=device).reshape(E, 1)
+    tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+    gate, dy = pr["gate"], pr["dy"]
+    full, irg, p1c = ops.cvmm_bwd_x(dy, pr["values"], offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
+                                    ir=ir_dn, ir_by_expert=True, relu_mask=True, decay=0.01, want_xc=True)
+    full2, irg2 = ops.cvmm_bwd_x(dy, pr["values"], offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
+                                 ir=ir_dn, ir_by_expert=True, relu_mask=True, decay=0.01)
+    assert torch.equal(full, full2) and torch.equal(irg, irg2)
+    ir_rows = ir_dn[pr["idx"].reshape(-1).long()]
+    want = (torch.minimum(torch.maximum(p1.float(), -ir_rows), ir_rows) * gate.reshape(-1, 1).float()).to(dtype)
+    assert torch.equal(p1c, want)
+    a = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
+    b = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, ir_by_expert=True, g_scale=gate)
+    assert torch.equal(a, b)
