@@ -56,18 +56,27 @@ class AnalogMoEFFN(torch.autograd.Function):
         E, _, F = keys.shape
         k = sel_idx.shape[-1]
         M = T * k
+        gen = cfg.noise_std > 0 and cfg.noise_up is None
+        wu = wd = None
+        main = torch.cuda.current_stream()
+        if cfg.out_bound > 0 or gen:
+            # max |W| per expert only reads the weights: it runs next to the expert sort on a second stream
+            side = _side_stream(x.device)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
+                wd = ops.weight_abs_max(values, cfg.noise_per_channel)
+            wu.record_stream(main)
+            wd.record_stream(main)
         sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
+        if wu is not None:
+            main.wait_stream(side)
         ntu = 1 if cfg.bounds_up is None else len(cfg.bounds_up) - 1
         ntd = 1 if cfg.bounds_down is None else len(cfg.bounds_down) - 1
         ir_up = ir_dn = None
         if input_range is not None:
             ir3 = input_range.detach().float().reshape(2, E, -1)
             ir_up, ir_dn = ir3[0, :, :ntu].contiguous(), ir3[1, :, :ntd].contiguous()
-        gen = cfg.noise_std > 0 and cfg.noise_up is None
-        wu = wd = None
-        if cfg.out_bound > 0 or gen:
-            wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
-            wd = ops.weight_abs_max(values, cfg.noise_per_channel)
         common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
                       noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
         # the up-projection also emits the down-projection's DAC image of its result (each row belongs
@@ -105,19 +114,21 @@ class AnalogMoEFFN(torch.autograd.Function):
         gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
                                           ir=ir_dn, bounds=cfg.bounds_down, relu_mask=True, want_xc=True,
                                           **irkw, **by)
-        # the gate gradient only streams z and dy through HBM; it runs on a second stream next to the
-        # weight gradient, whose workgroups leave registers and wave slots free on every CU
+        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
+                                      bounds=cfg.bounds_up, **irkw, **by)
+        # the gate gradient and the sum over the k heads only stream z, dy and the per-head input gradient
+        # through HBM; they run on a second stream next to the two weight gradients, whose workgroups
+        # leave registers and wave slots free on every CU
         main, side = torch.cuda.current_stream(), _side_stream(x.device)
         side.wait_stream(main)
         with torch.cuda.stream(side):
             grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+            grad_x = ops.ksum(full, k) if k > 1 else full
         grad_gate.record_stream(main)
+        grad_x.record_stream(main)
         grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
         grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
         main.wait_stream(side)
-        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
-                                      bounds=cfg.bounds_up, **irkw, **by)
-        grad_x = ops.ksum(full, k) if k > 1 else full
         grad_ir = None
         if ir_up is not None and ctx.needs_input_grad[3]:
             ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
