@@ -260,12 +260,14 @@ __device__ __host__ inline NoiseKey noise_key(uint64_t seed, int tile) {
   k.seed_hi = (uint32_t)(seed >> 32);
   return k;
 }
-__device__ __forceinline__ void noise_pair(const NoiseKey& key, uint64_t pair_ctr, float& z0, float& z1) {
-  uint32_t h = (uint32_t)pair_ctr ^ key.ka ^ ((uint32_t)(pair_ctr >> 32) * 0xC2B2AE3Du);
+// Key of an output row (once per row and K tile), then the pair of normals of column pair p.
+__device__ __forceinline__ uint32_t noise_row_key(const NoiseKey& key, uint32_t row) { return fmix32(row ^ key.ka); }
+__device__ __forceinline__ void noise_pair(const NoiseKey& key, uint32_t row_key, uint32_t pair, float& z0, float& z1) {
+  uint32_t h = row_key + pair * 0x9E3779B9u;
   h ^= h >> 16; h *= 0x85EBCA6Bu; h += key.kb; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
-  float u1 = ((float)(h >> 16) + 0.5f) * (1.0f / 65536.0f);
-  float u2 = ((float)(h & 0xffffu) + 0.5f) * (1.0f / 65536.0f);
-  float r = fast_sqrt(-1.3862943611f * fast_log2(u1));     // sqrt(-2 ln u1)
+  const float u1 = fmaf((float)(h >> 16), 1.0f / 65536.0f, 0.5f / 65536.0f);   // exact: (b + 0.5) / 65536
+  const float u2 = (float)(h & 0xffffu) * (1.0f / 65536.0f);
+  const float r = fast_sqrt(-1.3862943611f * fast_log2(u1));     // sqrt(-2 ln u1)
   z0 = r * fast_cos_rev(u2);
   z1 = r * fast_sin_rev(u2);
 }

@@ -229,7 +229,17 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 
     // per-column constants of the forward epilogue (last read before the barrier that ended the
     // previous item)
-    if (FWD && tid < kTileCols) {
+    // (with one max |W| per expert they are the same for every column: scalars, no LDS traffic)
+    const bool col_uniform = FWD && p.wmax_cols <= 1;
+    float u_nz = 0.f, u_bound = 0.f, u_q = 0.f, u_qinv = 0.f;
+    if (col_uniform) {
+      const float wm = p.wmax != nullptr ? p.wmax[(int64_t)e * p.wmax_cols] : 1.f;
+      u_nz = p.noise_std * wm;
+      u_bound = p.out_bound * wm;
+      u_q = adc_quant ? p.out_half_states / u_bound : 0.f;
+      u_qinv = adc_quant ? u_bound / p.out_half_states : 0.f;
+    }
+    if (FWD && !col_uniform && tid < kTileCols) {
       const int col = c0 + tid;
       float wm = 1.f;
       if (p.wmax != nullptr && col < c1) wm = p.wmax[(int64_t)e * p.wmax_cols + (p.wmax_cols > 1 ? col : 0)];
@@ -462,6 +472,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           const int orow = valid ? sOrow[rl] : 0;
           const float ir_r = (has_ir && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
           const float am_r = (has_amax && valid) ? p.abs_max[p.a_index[r]] : 1.f;
+          const uint32_t row_key = gen_noise ? noise_row_key(key, (uint32_t)orow) : 0u;
 #pragma unroll
           for (int fi = 0; fi < 2; fi++) {
 #pragma unroll
@@ -486,13 +497,18 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
                 for (int j = 0; j < 4; j++) v[j] += nz[j];
               } else if (gen_noise) {
                 float z[4];
-                const uint64_t ctr = (uint64_t)orow * (uint64_t)(p.ND >> 1) + (uint64_t)(col >> 1);
-                noise_pair(key, ctr, z[0], z[1]);
-                noise_pair(key, ctr + 1, z[2], z[3]);
+                noise_pair(key, row_key, (uint32_t)(col >> 1), z[0], z[1]);
+                noise_pair(key, row_key, (uint32_t)(col >> 1) + 1u, z[2], z[3]);
 #pragma unroll
-                for (int j = 0; j < 4; j++) v[j] += sCol[0][cl + j] * z[j];
+                for (int j = 0; j < 4; j++) v[j] += (col_uniform ? u_nz : sCol[0][cl + j]) * z[j];
               }
-              if (adc_clip) {
+              if (adc_clip && col_uniform) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  v[j] = clamp_sym(v[j], u_bound);
+                  if (adc_quant) v[j] = rintf(v[j] * u_q) * u_qinv;
+                }
+              } else if (adc_clip) {
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                   const float b = sCol[1][cl + j];

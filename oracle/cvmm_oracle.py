@@ -169,21 +169,20 @@ def counter_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.nda
     """Standard-normal noise for output rows ``rows`` (output-row ids), all ``n_cols``
     columns, K-tile ``tile``; a pure function of (seed, tile, row, column).
 
-    Columns are paired (2p, 2p+1) and the pair has the 64-bit counter ``row * n_cols/2 + p``.
-    Two 32-bit keys come from the seed halves and the tile; the counter is whitened with the
-    first key, run through the two multiply / xor-shift rounds of the murmur3 finaliser with
-    the second key added between them, and the 16-bit halves of the result give (u1, u2) in
-    (0,1); Box-Muller gives the pair (r cos 2 pi u2, r sin 2 pi u2), r = sqrt(-2 ln u1).
-    n_cols must be even."""
+    Columns are paired (2p, 2p+1).  Two 32-bit keys come from the seed halves and the tile.  The
+    row gets the key ``fmix32(row ^ ka)``; the pair's word is that key plus ``p * 0x9E3779B9``,
+    run through the two multiply / xor-shift rounds of the murmur3 finaliser with the second key
+    added between them; the 16-bit halves of the result give u1 in (0,1) and u2 in [0,1);
+    Box-Muller gives the pair (r cos 2 pi u2, r sin 2 pi u2), r = sqrt(-2 ln u1).
+    n_cols must be even; rows and pair indices are taken modulo 2**32."""
     assert n_cols % 2 == 0
-    rows = np.asarray(rows, dtype=np.uint64).reshape(-1, 1)
+    rows = _u32(np.asarray(rows, dtype=np.uint64)).reshape(-1, 1)
     p = np.arange(n_cols // 2, dtype=np.uint64).reshape(1, -1)
-    ctr = rows * np.uint64(n_cols // 2) + p
-    lo, hi = _u32(ctr), _u32(ctr >> np.uint64(32))
     s_lo, s_hi = seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF
     ka = _fmix32(_u32((s_lo ^ 0x9E3779B9) + tile * 0x632BE5AB))
     kb = _fmix32(_u32((s_hi ^ 0x85EBCA77) + tile * 0x27D4EB2F))
-    h = lo ^ ka ^ _u32(hi.astype(np.uint64) * np.uint64(0xC2B2AE3D))
+    row_key = _fmix32(rows ^ ka)
+    h = _u32(row_key.astype(np.uint64) + p * np.uint64(0x9E3779B9))
     h ^= h >> np.uint32(16)
     h = _u32(h.astype(np.uint64) * np.uint64(0x85EBCA6B))
     h = _u32(h.astype(np.uint64) + np.uint64(kb))
@@ -191,7 +190,7 @@ def counter_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.nda
     h = _u32(h.astype(np.uint64) * np.uint64(0xC2B2AE35))
     h ^= h >> np.uint32(16)
     u1 = ((h >> np.uint32(16)).astype(F32) + F32(0.5)) * F32(1.0 / 65536.0)
-    u2 = ((h & np.uint32(0xFFFF)).astype(F32) + F32(0.5)) * F32(1.0 / 65536.0)
+    u2 = (h & np.uint32(0xFFFF)).astype(F32) * F32(1.0 / 65536.0)
     r = np.sqrt(F32(-2.0) * np.log(u1.astype(np.float64)))
     ang = 2.0 * np.pi * u2.astype(np.float64)
     out = np.empty((rows.shape[0], n_cols), dtype=F32)
