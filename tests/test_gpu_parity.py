@@ -158,3 +158,65 @@ def test_chained_projections(ops, dtype, D, F):
                                        (torch.bfloat16, 72, 40)])
 def test_clipped_input_for_the_weight_gradient(ops, dtype, D, F):
     util.check_clipped_input_output(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)
+
+
+@pytest.mark.parametrize("name,T,D,E,F,k,routing", [("config3", 16384, 1024, 64, 256, 8, "uniform"),
+                                                     ("config4", 32768, 2048, 128, 512, 4, "zipf")])
+def test_full_size_properties(ops, name, T, D, E, F, k, routing):
+    """BASELINE configs 3 and 4 at full size (bf16), where the oracle is too slow to run whole: sampled
+    rows of both forward projections against float64 arithmetic on the kernel's own DAC definition,
+    token-permutation invariance (bit-exact), run-to-run identity and exact power-of-two scaling of the
+    weight gradient, and the sort invariants."""
+    print(name, flush=True)
+    pr = _to(util.make_problem(0, T, D, E, F, k, dtype=torch.bfloat16, routing=routing))
+    x, keys, values, idx, dy = pr["x"], pr["keys"], pr["values"], pr["idx"], pr["dy"]
+    M = T * k
+    ss, perm, in_index, offsets = ops.prepare_sel(idx, E, k)
+    flat = idx.reshape(-1)
+    assert torch.equal(flat[perm.long()].int(), ss) and bool((ss[1:] >= ss[:-1]).all())
+    assert torch.equal(offsets.long(), torch.cat([torch.zeros(1, dtype=torch.long, device="cuda"),
+                                                  torch.bincount(flat, minlength=E).cumsum(0)]))
+    assert torch.equal(in_index, (perm // k).int())
+    res = 1 / 127
+    ir_up = torch.linspace(2.0, 3.5, E, device="cuda").reshape(E, 1)
+    ir_dn = torch.linspace(1.0, 2.0, E, device="cuda").reshape(E, 1)
+    fwd_up = lambda xx, ii, oo: ops.cvmm_fwd(xx, keys, ss, offsets, ii, oo, M, ir=ir_up, ir_by_expert=True,
+                                             inp_res=res, relu=True)
+    p1 = fwd_up(x, in_index, perm)
+    z = ops.cvmm_fwd(p1, values, ss, offsets, perm, None, M, ir=ir_dn, ir_by_expert=True, inp_res=res)
+    # sampled sorted positions against float64 (codes are exact in bf16; weights are the bf16 values)
+    g = torch.Generator().manual_seed(1)
+    pos = torch.randint(0, M, (192,), generator=g).cuda()
+    e_of = ss[pos].long()
+
+    def ref_rows(inp_rows, w, ir_tab):
+        r = ir_tab[e_of].double()
+        a = torch.minimum(torch.maximum(inp_rows.double(), -r), r)
+        a32 = (a.float() / r.float())                       # fp32 divisions, as the kernel does them
+        codes = torch.round(a32 / torch.tensor(res, dtype=torch.float32, device="cuda"))
+        out = torch.einsum("rk,rkn->rn", codes.double(), w[e_of].double()) * float(np.float32(res))
+        return out * r
+
+    want_p1 = torch.relu(ref_rows(x[in_index[pos].long()], keys, ir_up))
+    got_p1 = p1[perm[pos].long()].double()
+    assert float((got_p1 - want_p1).abs().max() / want_p1.abs().max()) < 1e-2          # bf16 output rounding
+    want_z = ref_rows(p1[perm[pos].long()], values, ir_dn)
+    got_z = z[perm[pos].long()].double()
+    assert float((got_z - want_z).abs().max() / want_z.abs().max()) < 1e-2
+    # shuffling the tokens permutes the outputs identically, bit for bit
+    shuf = torch.randperm(T, generator=g).cuda()
+    idx2 = idx[shuf]
+    ss2, perm2, in2, off2 = ops.prepare_sel(idx2, E, k)
+    p1_2 = ops.cvmm_fwd(x[shuf], keys, ss2, off2, in2, perm2, M, ir=ir_up, ir_by_expert=True, inp_res=res, relu=True)
+    assert torch.equal(p1_2.view(T, k, F), p1.view(T, k, F)[shuf])
+    # weight gradient: identical from run to run, and exactly linear under a power-of-two scale
+    tok = (perm // k).int()
+    gw = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, ir_by_expert=True)
+    assert torch.equal(gw, ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, ir_by_expert=True))
+    gw4 = ops.cvmm_bwd_w(p1, dy * 4, E, offsets, perm, tok, ir=ir_dn, ir_by_expert=True)
+    assert torch.equal(gw4, gw * 4)
+    # input gradient of the plain product against float64 on the sampled rows
+    full, _ = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M)
+    want_g = torch.einsum("rn,rkn->rk", dy[tok[pos].long()].double(), values[e_of].double())
+    got_g = full[perm[pos].long()].double()
+    assert float((got_g - want_g).abs().max() / want_g.abs().max()) < 1e-2
