@@ -35,8 +35,8 @@ CONFIGS = {
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
 # the counter runs summarised under profiles/; None where not measured
-TRAFFIC = {"c3": {"fwd_up": 431599230, "fwd_down": 452181449, "wgrad_down": 370379901, "wgrad_up": 370405273,
-                  "xgrad_down": 477040965, "xgrad_up": 695967656}}
+TRAFFIC = {"c3": {"fwd_up": 449264702, "fwd_down": 452088530, "wgrad_down": 370375802, "wgrad_up": 370387608,
+                  "xgrad_down": 479622544, "xgrad_up": 695208049}}
 
 
 def cpu_baseline(cfg, pr, budget_tokens):
