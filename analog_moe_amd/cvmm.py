@@ -13,7 +13,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from . import ops
+from . import library  # noqa: F401  (registers the amoe:: operators used below)
 from .config import enum_name
 
 
@@ -33,7 +33,7 @@ class CVMMSel:
 
 def cvmm_prepare_sel(sel: torch.Tensor, n_experts: int) -> CVMMSel:
     """cvmm.py:31-34: sorted ids and the permutation; ties keep ascending flat index."""
-    ssel, perm, _, offsets = ops.prepare_sel(sel, n_experts, 1)
+    ssel, perm, _, offsets = torch.ops.amoe.prepare_sel(sel, n_experts, 1)
     return CVMMSel(sel, ssel.view(sel.shape), perm, None, None, offsets)
 
 
@@ -41,15 +41,15 @@ def cvmm_prepare_sel2(sel: torch.Tensor, n_experts: int, w: Optional[torch.Tenso
     """Selection record of a k-head layer as the up-projection uses it: ``sel_index = perm // k``
     (token row), ``out_index = perm`` (cvmm.py:196-205, 828-833)."""
     k = sel.shape[-1]
-    ssel, perm, in_index, offsets = ops.prepare_sel(sel, n_experts, k)
+    ssel, perm, in_index, offsets = torch.ops.amoe.prepare_sel(sel, n_experts, k)
     return CVMMSel(sel, ssel.view(sel.shape), in_index, perm, w, offsets)
 
 
 def cvmm_std(x: torch.Tensor, sel_index: torch.Tensor, sel: torch.Tensor, n_experts: int) -> torch.Tensor:
     """Per-expert unbiased std of the routed rows' elements (cvmm.py:400-443)."""
     ssel = sel.reshape(-1).to(torch.int32)
-    offsets = ops.offsets_from_sorted(ssel, n_experts)
-    return ops.expert_std(x, sel_index, offsets, n_experts).to(x.dtype)
+    offsets = torch.ops.amoe.offsets_from_sorted(ssel, n_experts)
+    return torch.ops.amoe.expert_std(x, sel_index.to(torch.int32), offsets, n_experts).to(x.dtype)
 
 
 @dataclass
@@ -62,7 +62,7 @@ class AnalogExt:
     out_res: float = -1.0
     noise_std: float = 0.0                       # generate noise in the kernel from noise_seed
     noise_seed: int = 0
-    noise_seed_dev: Optional[Tensor] = None      # int64 device word added to the seed by the kernel
+    noise_seed_dev: Optional[torch.Tensor] = None      # int64 device word added to the seed by the kernel
 
 
 def _abs_max_wanted(ir_params, io_params) -> bool:
@@ -74,6 +74,9 @@ def _abs_max_wanted(ir_params, io_params) -> bool:
 
 
 class CVMM(torch.autograd.Function):
+    """cvmm.py:699-897.  The launches sit behind the operators ``amoe::cvmm_forward`` and
+    ``amoe::cvmm_backward``; what is left here is shape and dtype glue that ``torch.compile`` can trace."""
+
     @staticmethod
     def forward(ctx, x, sel_index, sel, keys, inp_res, broadcasted_input_ranges=None, out_index=None,
                 reduction_weight=None, out_noise=None, ir_params=None, io_params=None, ext=None):
@@ -87,69 +90,46 @@ class CVMM(torch.autograd.Function):
         else:
             keys_op = keys if keys.dtype == x.dtype else keys.to(x.dtype)
         ssel = sel.reshape(-1).to(torch.int32)
-        offsets = ext.offsets if ext.offsets is not None else ops.offsets_from_sorted(ssel, E)
+        offsets = ext.offsets if ext.offsets is not None else torch.ops.amoe.offsets_from_sorted(ssel, E)
         sel_index = sel_index.to(torch.int32)
         out_index = None if out_index is None else out_index.to(torch.int32)
-        abs_max = ops.row_abs_max(x) if _abs_max_wanted(ir_params, io_params) else None
         M = ssel.numel()
-        n_tiles = 1 if ext.bounds is None else len(ext.bounds) - 1
+        bounds = None if ext.bounds is None else list(ext.bounds)
+        n_tiles = 1 if bounds is None else len(bounds) - 1
         bir = None
         if broadcasted_input_ranges is not None:
             bir = broadcasted_input_ranges.detach().reshape(M, n_tiles).float().contiguous()
         noise = None
         if out_noise is not None:
             noise = out_noise.detach().float().reshape(n_tiles, M, N).contiguous()
-        res = ops.cvmm_fwd(x, keys_op, ssel, offsets, sel_index, out_index, M, ir=bir, abs_max=abs_max,
-                           inp_res=float(inp_res), bounds=ext.bounds, noise=noise, noise_std=ext.noise_std,
-                           noise_seed=ext.noise_seed, noise_seed_dev=ext.noise_seed_dev, wmax=ext.wmax, out_bound=ext.out_bound,
-                           out_res=ext.out_res)
-        res = res.view(*sel.shape, N)
-        z = None
-        if reduction_weight is not None:                     # cvmm.py:757-759
-            z = res
-            res = ops.gate_reduce(z, reduction_weight).view(*reduction_weight.shape[:-1], N)
-        ctx.save_for_backward(x, keys_op, ssel, sel_index, out_index, reduction_weight, bir, z, offsets)
-        ctx.ir_params = ir_params
+        gate = None if reduction_weight is None else reduction_weight.detach()
+        res, z = torch.ops.amoe.cvmm_forward(
+            x, keys_op, ssel, offsets, sel_index, out_index, gate, bir, noise, _abs_max_wanted(ir_params, io_params),
+            float(inp_res), bounds, ext.wmax, float(ext.out_bound), float(ext.out_res), float(ext.noise_std),
+            int(ext.noise_seed), ext.noise_seed_dev)
+        if reduction_weight is None:
+            res, z = res.view(*sel.shape, N), None
+        else:                                                   # cvmm.py:757-759
+            res, z = res.view(*reduction_weight.shape[:-1], N), z.view(*sel.shape, N)
+        ctx.save_for_backward(x, keys_op, sel_index, out_index, reduction_weight, bir, z, offsets)
+        ctx.ir_grad_args = (bool(getattr(ir_params, "gradient_relative", True)),
+                            float(getattr(ir_params, "gradient_scale", 1.0)),
+                            float(getattr(ir_params, "decay", 0.0)),
+                            float(getattr(ir_params, "input_min_percentage", 0.95)))
         ctx.bir_shape = None if broadcasted_input_ranges is None else broadcasted_input_ranges.shape
         ctx.bir_dtype = None if broadcasted_input_ranges is None else broadcasted_input_ranges.dtype
-        ctx.bounds = ext.bounds
+        ctx.bounds = bounds
         ctx.keys_dtype = keys.dtype
-        ctx.x_shape = x.shape
         return res
 
     @staticmethod
     def backward(ctx, grad_output):
-        x, keys, ssel, sel_index, out_index, gate, bir, z, offsets = ctx.saved_tensors
-        ir_params = ctx.ir_params
-        E, K, N = keys.shape
-        M = ssel.numel()
-        grad_output = grad_output.to(x.dtype).contiguous()
-        pos_out = sel_index if out_index is None else out_index        # cvmm.py:828
-        irkw = {}
-        if bir is not None:
-            irkw = dict(gradient_relative=getattr(ir_params, "gradient_relative", True),
-                        gradient_scale=getattr(ir_params, "gradient_scale", 1.0),
-                        decay=getattr(ir_params, "decay", 0.0),
-                        input_min_percentage=getattr(ir_params, "input_min_percentage", 0.95))
-        if gate is not None:
-            k = gate.shape[-1]
-            g_rows = torch.div(pos_out, k, rounding_mode="floor").to(torch.int32)   # cvmm.py:833
-            grad_w = ops.cvmm_bwd_w(x, grad_output, E, offsets, sel_index, g_rows, ir=bir, bounds=ctx.bounds,
-                                    g_scale=gate)                                    # cvmm.py:785-789, 812-823
-            full, ir_grad = ops.cvmm_bwd_x(grad_output, keys, offsets, g_rows, pos_out, M, x=x,
-                                           xf_index=sel_index, gate=gate, ir=bir, bounds=ctx.bounds, **irkw)
-            grad_x = full.view(ctx.x_shape)                                          # cvmm.py:888
-            grad_gate = ops.gate_grad(z, grad_output, k).view(gate.shape).to(gate.dtype)  # cvmm.py:889
-        else:
-            grad_w = ops.cvmm_bwd_w(x, grad_output, E, offsets, sel_index, out_index, ir=bir, bounds=ctx.bounds)
-            full, ir_grad = ops.cvmm_bwd_x(grad_output, keys, offsets, pos_out, pos_out, M, x=x,
-                                           xf_index=sel_index, ir=bir, bounds=ctx.bounds, **irkw)
-            k = M // max(x.reshape(-1, K).shape[0], 1)
-            grad_x = (ops.ksum(full, k) if k > 1 else full).view(ctx.x_shape)        # cvmm.py:890-893
-            grad_gate = None
-        if ir_grad is not None and ctx.needs_input_grad[5]:
+        x, keys, sel_index, out_index, gate, bir, z, offsets = ctx.saved_tensors
+        grad_x, grad_w, ir_grad, grad_gate = torch.ops.amoe.cvmm_backward(
+            grad_output, x, keys, offsets, sel_index, out_index, gate, bir, z, ctx.bounds, *ctx.ir_grad_args)
+        if bir is not None and ctx.needs_input_grad[5]:
             ir_grad = ir_grad.view(ctx.bir_shape).to(ctx.bir_dtype)       # cvmm.py:897
         else:
             ir_grad = None
-        return (grad_x, None, None, grad_w.to(ctx.keys_dtype), None, ir_grad, None, grad_gate, None, None, None,
-                None)
+        return (grad_x, None, None, grad_w.to(ctx.keys_dtype), None, ir_grad, None,
+                None if gate is None else grad_gate, None, None, None, None)

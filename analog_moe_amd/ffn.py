@@ -46,51 +46,116 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
     return _SIDE_STREAMS[key]
 
 
+CFG_FIELDS = ("inp_res", "bounds_up", "bounds_down", "out_bound", "out_res", "noise_std", "noise_seed",
+              "noise_seed_dev", "noise_per_channel", "gradient_relative", "gradient_scale", "decay",
+              "input_min_percentage", "noise_up", "noise_down")
+
+
+def cfg_astuple(cfg: FFNConfig) -> tuple:
+    """The configuration as positional values, in the order the ``amoe::ffn_fwd`` operator takes them."""
+    return tuple(getattr(cfg, f) for f in CFG_FIELDS)
+
+
+def _n_tiles(bounds) -> int:
+    return 1 if bounds is None else len(bounds) - 1
+
+
+def ir_tables(input_range: Optional[torch.Tensor], E: int, cfg: FFNConfig):
+    """Per-expert input ranges of the two projections, fp32: [E, n_tiles_up], [E, n_tiles_down]."""
+    if input_range is None:
+        return None, None
+    ir3 = input_range.detach().float().reshape(2, E, -1)
+    return ir3[0, :, :_n_tiles(cfg.bounds_up)].contiguous(), ir3[1, :, :_n_tiles(cfg.bounds_down)].contiguous()
+
+
+def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
+    """Sort, both projections and the gate reduction.  Returns (y, p1, z, perm, in_index, offsets, ir_up,
+    ir_dn): the result and what the backward pass reads again."""
+    T, D = x.shape
+    E, _, F = keys.shape
+    k = sel_idx.shape[-1]
+    M = T * k
+    gen = cfg.noise_std > 0 and cfg.noise_up is None
+    wu = wd = None
+    main = torch.cuda.current_stream()
+    if cfg.out_bound > 0 or gen:
+        # max |W| per expert only reads the weights: it runs next to the expert sort on a second stream
+        side = _side_stream(x.device)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
+            wd = ops.weight_abs_max(values, cfg.noise_per_channel)
+        wu.record_stream(main)
+        wd.record_stream(main)
+    sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
+    if wu is not None:
+        main.wait_stream(side)
+    ir_up, ir_dn = ir_tables(input_range, E, cfg)
+    common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
+                  noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
+    # the up-projection also emits the down-projection's DAC image of its result (each row belongs
+    # to one expert, so the image is made once instead of once per block of output columns)
+    chain = ir_dn is not None and cfg.inp_res > 0 and _n_tiles(cfg.bounds_down) == 1
+    p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, bounds=cfg.bounds_up,
+                      noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True,
+                      noise_seed_dev=cfg.noise_seed_dev, xq_ir=ir_dn[:, 0].contiguous() if chain else None,
+                      xq_inp_res=cfg.inp_res, **common)
+    p1, p1q = p1 if chain else (p1, None)
+    z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn,
+                     bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
+                     noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
+    y = ops.gate_reduce(z, gate)
+    return y, p1, z, perm, in_index, offsets, ir_up, ir_dn
+
+
+def ffn_backward(dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn, cfg: FFNConfig,
+                 want_ir_grad: bool):
+    """Returns (grad_x, grad_keys, grad_values, grad_ir [2, E, n_tiles] fp32 or None, grad_gate)."""
+    E = keys.shape[0]
+    k = gate.shape[-1]
+    M = perm.numel()
+    dy = dy.contiguous()
+    by = dict(ir_by_expert=ir_up is not None)
+    irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
+                input_min_percentage=cfg.input_min_percentage)
+    tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+    # the input gradient reads p1 for its masks anyway; it also leaves gate * clamp(p1), which is the
+    # x operand of the weight gradient (otherwise every block of its output columns clips and scales)
+    gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
+                                      ir=ir_dn, bounds=cfg.bounds_down, relu_mask=True, want_xc=True,
+                                      **irkw, **by)
+    full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
+                                  bounds=cfg.bounds_up, **irkw, **by)
+    # the gate gradient and the sum over the k heads only stream z, dy and the per-head input gradient
+    # through HBM; they run on a second stream next to the two weight gradients, whose workgroups
+    # leave registers and wave slots free on every CU
+    main, side = torch.cuda.current_stream(), _side_stream(x.device)
+    side.wait_stream(main)
+    with torch.cuda.stream(side):
+        grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+        grad_x = ops.ksum(full, k) if k > 1 else full
+    grad_gate.record_stream(main)
+    grad_x.record_stream(main)
+    grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
+    grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
+    main.wait_stream(side)
+    grad_ir = None
+    if ir_up is not None and want_ir_grad:
+        ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
+        grad_ir = torch.zeros((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
+        grad_ir[0, :, :ntu] = ops.segment_sum(irg_up, offsets, E)
+        grad_ir[1, :, :ntd] = ops.segment_sum(irg_dn, offsets, E)
+    return grad_x, grad_keys, grad_values, grad_ir, grad_gate
+
+
 class AnalogMoEFFN(torch.autograd.Function):
     """y[t] = sum_j gate[t,j] * A(relu(A(x[t], keys[e_tj])), values[e_tj]).
     input_range: [2, E, n_tiles] (row 0 up-, row 1 down-projection) or None."""
 
     @staticmethod
     def forward(ctx, x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
-        T, D = x.shape
-        E, _, F = keys.shape
-        k = sel_idx.shape[-1]
-        M = T * k
-        gen = cfg.noise_std > 0 and cfg.noise_up is None
-        wu = wd = None
-        main = torch.cuda.current_stream()
-        if cfg.out_bound > 0 or gen:
-            # max |W| per expert only reads the weights: it runs next to the expert sort on a second stream
-            side = _side_stream(x.device)
-            side.wait_stream(main)
-            with torch.cuda.stream(side):
-                wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
-                wd = ops.weight_abs_max(values, cfg.noise_per_channel)
-            wu.record_stream(main)
-            wd.record_stream(main)
-        sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
-        if wu is not None:
-            main.wait_stream(side)
-        ntu = 1 if cfg.bounds_up is None else len(cfg.bounds_up) - 1
-        ntd = 1 if cfg.bounds_down is None else len(cfg.bounds_down) - 1
-        ir_up = ir_dn = None
-        if input_range is not None:
-            ir3 = input_range.detach().float().reshape(2, E, -1)
-            ir_up, ir_dn = ir3[0, :, :ntu].contiguous(), ir3[1, :, :ntd].contiguous()
-        common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
-                      noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
-        # the up-projection also emits the down-projection's DAC image of its result (each row belongs
-        # to one expert, so the image is made once instead of once per block of output columns)
-        chain = ir_dn is not None and cfg.inp_res > 0 and ntd == 1
-        p1 = ops.cvmm_fwd(x, keys, sel_sorted, offsets, in_index, perm, M, ir=ir_up, bounds=cfg.bounds_up,
-                          noise=cfg.noise_up, noise_seed=cfg.noise_seed, wmax=wu, relu=True,
-                          noise_seed_dev=cfg.noise_seed_dev, xq_ir=ir_dn[:, 0].contiguous() if chain else None,
-                          xq_inp_res=cfg.inp_res, **common)
-        p1, p1q = p1 if chain else (p1, None)
-        z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn,
-                         bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
-                         noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
-        y = ops.gate_reduce(z, gate)
+        y, p1, z, perm, in_index, offsets, ir_up, ir_dn = ffn_forward(x, keys, values, input_range, gate,
+                                                                      sel_idx, cfg)
         ctx.save_for_backward(x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn)
         ctx.cfg = cfg
         ctx.ir_shape = None if input_range is None else input_range.shape
@@ -100,40 +165,18 @@ class AnalogMoEFFN(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn = ctx.saved_tensors
-        cfg = ctx.cfg
-        E = keys.shape[0]
-        k = gate.shape[-1]
-        M = perm.numel()
-        dy = dy.contiguous()
-        by = dict(ir_by_expert=ir_up is not None)
-        irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
-                    input_min_percentage=cfg.input_min_percentage)
-        tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
-        # the input gradient reads p1 for its masks anyway; it also leaves gate * clamp(p1), which is the
-        # x operand of the weight gradient (otherwise every block of its output columns clips and scales)
-        gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
-                                          ir=ir_dn, bounds=cfg.bounds_down, relu_mask=True, want_xc=True,
-                                          **irkw, **by)
-        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
-                                      bounds=cfg.bounds_up, **irkw, **by)
-        # the gate gradient and the sum over the k heads only stream z, dy and the per-head input gradient
-        # through HBM; they run on a second stream next to the two weight gradients, whose workgroups
-        # leave registers and wave slots free on every CU
-        main, side = torch.cuda.current_stream(), _side_stream(x.device)
-        side.wait_stream(main)
-        with torch.cuda.stream(side):
-            grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
-            grad_x = ops.ksum(full, k) if k > 1 else full
-        grad_gate.record_stream(main)
-        grad_x.record_stream(main)
-        grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
-        grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
-        main.wait_stream(side)
-        grad_ir = None
-        if ir_up is not None and ctx.needs_input_grad[3]:
-            ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
-            gi = torch.zeros((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
-            gi[0, :, :ntu] = ops.segment_sum(irg_up, offsets, E)
-            gi[1, :, :ntd] = ops.segment_sum(irg_dn, offsets, E)
-            grad_ir = gi.reshape(ctx.ir_shape).to(ctx.ir_dtype)
+        grad_x, grad_keys, grad_values, grad_ir, grad_gate = ffn_backward(
+            dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn, ctx.cfg,
+            ctx.needs_input_grad[3])
+        if grad_ir is not None:
+            grad_ir = grad_ir.reshape(ctx.ir_shape).to(ctx.ir_dtype)
         return grad_x, grad_keys, grad_values, grad_ir, grad_gate, None, None
+
+
+def moe_ffn(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig) -> torch.Tensor:
+    """The fused expert feed-forward.  Eagerly this is ``AnalogMoEFFN``; while ``torch.compile`` traces,
+    the same two functions are reached through the opaque operators ``amoe::ffn_fwd`` / ``amoe::ffn_bwd``
+    (their side streams and ctypes calls are nothing a tracer can follow)."""
+    if torch.compiler.is_compiling():
+        return torch.ops.amoe.ffn_fwd(x, keys, values, input_range, gate, sel_idx, *cfg_astuple(cfg))[0]
+    return AnalogMoEFFN.apply(x, keys, values, input_range, gate, sel_idx, cfg)

@@ -24,10 +24,10 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from . import ops
 from .config import (TorchInferenceRPUConfig, WeightClipType, WeightModifierType, enum_name, kernel_inp_res)
 from .cvmm import CVMM, AnalogExt, CVMMSel, cvmm_prepare_sel2, cvmm_std
-from .ffn import AnalogMoEFFN, FFNConfig
+from . import library  # noqa: F401  (registers the amoe:: operators)
+from .ffn import FFNConfig, moe_ffn
 
 
 class MoEConifgError(Exception):
@@ -132,7 +132,7 @@ class SigmaMoELayer(nn.Module):
 
     def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
         """Expert feed-forward for a given routing decision (what follows the router in forward)."""
-        if not x.is_cuda:
+        if not (x.is_cuda or x.is_meta):
             raise MoEConifgError("MoE layer executed on CPU: this package runs on the GPU only "
                                  "(moe_layer_aihwkit_lightning.py:395-400 raises the same way)")
         sel_indices = cvmm_prepare_sel2(sel_idx, self.n_experts)
@@ -193,6 +193,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             raise MoEConifgError("noise_mode must be 'kernel' or 'injected'")
         self.noise_mode = noise_mode
         self._noise_calls = 0
+        self._noise_seed_base = 0
         self._init_done = False            # host-side latch of "input_range_update_idx reached init_from_data"
         self.noise_counter: Optional[Tensor] = None     # see use_device_noise_counter()
         self._register_load_state_dict_pre_hook(load_state_dict_pre_hook)
@@ -322,20 +323,26 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     def use_device_noise_counter(self) -> Tensor:
         """Keep the per-call part of the noise seed in device memory (one int64 word that every noisy
         launch reads and every forward bumps on the stream).  A forward captured in a HIP graph then
-        draws new noise on each replay; without it the seed is a launch argument frozen at capture."""
+        draws new noise on each replay; without it the seed is a launch argument frozen at capture.  The
+        same holds for a forward traced by ``torch.compile``.  Calling this again re-reads torch's seed."""
         if self.noise_counter is None:
             self.noise_counter = torch.zeros(1, dtype=torch.int64, device=self.keys.device)
+        # the host part of the seed is read here, once: a traced or captured forward cannot ask for it
+        self._noise_seed_base = (torch.initial_seed() * 0x9E3779B97F4A7C15) & (2 ** 63 - 1)
         return self.noise_counter
 
     def _noise_seed(self) -> int:
         if self.noise_counter is not None:       # the call count lives on the device
-            return (torch.initial_seed() * 0x9E3779B97F4A7C15) & (2 ** 63 - 1)
+            return self._noise_seed_base
+        if torch.compiler.is_compiling():
+            raise MoEConifgError("a compiled noisy forward would freeze the host-side noise seed: call "
+                                 "use_device_noise_counter() on the layer before torch.compile")
         self._noise_calls += 1
         return (torch.initial_seed() * 0x9E3779B97F4A7C15 + self._noise_calls * 0xD1B54A32D192ED03) & (2 ** 63 - 1)
 
     def cvmm_wrapper(self, inputs: Tensor, sel_indices: CVMMSel, weights: Tensor) -> Tensor:
         """moe_layer_aihwkit_lightning.py:412-507."""
-        if not inputs.is_cuda:
+        if not (inputs.is_cuda or inputs.is_meta):
             raise MoEConifgError("Analog MoE executed on CPU. This package runs on the GPU only.")
         fwd = self.rpu_config.forward
         is_up = inputs.ndim == 3
@@ -360,7 +367,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         per_channel = bool(getattr(fwd, "out_noise_per_channel", False))
         noisy = self.training and fwd.out_noise > 0
         if ext.out_bound > 0 or noisy:
-            ext.wmax = ops.weight_abs_max(weights, per_channel)
+            ext.wmax = torch.ops.amoe.weight_abs_max(weights.detach(), per_channel)
         out_noise = None
         if noisy and self.noise_mode == "kernel":
             ext.noise_std, ext.noise_seed = float(fwd.out_noise), self._noise_seed()
@@ -382,7 +389,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
                 not (self.training and self._init_from_data_pending()))
 
     def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
-        if not x.is_cuda or not self._fusable():
+        if not (x.is_cuda or x.is_meta) or not self._fusable():
             return super().forward_selected(x, sel_val, sel_idx)
         fwd = self.rpu_config.forward
         irp = self.rpu_config.pre_post.input_range
@@ -400,15 +407,16 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             M = sel_idx.numel()
             flat = sel_idx.reshape(-1)
             pc = cfg.noise_per_channel
-            wu, wd = ops.weight_abs_max(self.keys, pc), ops.weight_abs_max(self.values, pc)
+            wu = torch.ops.amoe.weight_abs_max(self.keys.detach(), pc)
+            wd = torch.ops.amoe.weight_abs_max(self.values.detach(), pc)
             ntu = 1 if self.bounds_up is None else len(self.bounds_up) - 1
             ntd = 1 if self.bounds_down is None else len(self.bounds_down) - 1
             cfg.noise_up = torch.randn(ntu, M, self.expert_size, device=x.device) * fwd.out_noise * wu[flat]
             cfg.noise_down = torch.randn(ntd, M, self.v_dim, device=x.device) * fwd.out_noise * wd[flat]
         lead = x.shape[:-1]
-        y = AnalogMoEFFN.apply(x.reshape(-1, x.shape[-1]), self.keys.to(x.dtype), self.values.to(x.dtype),
-                               self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
-                               sel_idx.reshape(-1, self.n_heads), cfg)
+        y = moe_ffn(x.reshape(-1, x.shape[-1]), self.keys.to(x.dtype), self.values.to(x.dtype),
+                    self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
+                    sel_idx.reshape(-1, self.n_heads), cfg)
         if cfg.noise_seed_dev is not None:
             cfg.noise_seed_dev.add_(2)             # the two projections used seed + 0 and seed + 1
         y = y.view(*lead, self.v_dim)

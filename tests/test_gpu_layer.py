@@ -228,3 +228,53 @@ def test_layer_step_replays_from_a_hip_graph():
             assert torch.equal(g, w)
     assert not torch.equal(outs[0][0], outs[1][0])                      # new noise on every replay
     del saved
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_compiled_layer_equals_eager(fused):
+    """torch.compile (one graph, forward and backward) runs the same launches as the eager layer: with the
+    noise off the results are bit-identical."""
+    from analog_moe_amd import config as cfgmod
+    torch._dynamo.reset()
+    mods = {} if fused else {"bias": True}
+    layer = _layer(cfgmod, mods, decay=0.01, max_input_size=64, out_bound=12.0, out_res=254)
+    assert layer._fusable() == fused
+    layer.train()
+    x = torch.randn(6, 20, 128, device="cuda", requires_grad=True)
+    dy = torch.randn(6, 20, 128, device="cuda")
+    params = [x, layer.keys, layer.values, layer.input_range, layer.expert_sel.weight]
+
+    def run(fn):
+        for p in params:
+            p.grad = None
+        y, reg = fn(x)
+        (y * dy).sum().add(reg).backward()
+        return [y.detach().clone()] + [p.grad.clone() for p in params]
+
+    want = run(layer)
+    got = run(torch.compile(layer, backend="aot_eager", fullgraph=True))
+    for w, g in zip(want, got):
+        assert torch.equal(w, g)
+
+
+def test_reference_operator_matches_oracle():
+    """torch.ops.amoe.cvmm_quantized with the reference's calling convention (cvmm.py:531-631): a one-element
+    tensor of -1 stands for an absent argument."""
+    from analog_moe_amd.cvmm import cvmm_prepare_sel2
+    pr = util.make_problem(5, 96, 72, 5, 40, 2, dtype=torch.float32)
+    pr = {n: t.cuda() for n, t in pr.items()}
+    s = cvmm_prepare_sel2(pr["idx"].view(8, 12, 2), 5)
+    minus = torch.tensor([-1.0], device="cuda")
+    x = pr["x"].view(8, 12, 72)
+    ir = torch.rand(8, 12, 2, device="cuda") + 0.5
+    noise = torch.randn(8, 12, 2, 40, device="cuda") * 0.01
+    want_sel = O.prepare_sel(pr["idx"].cpu().numpy(), 5, 2)
+    for ir_t, noise_t, inp_res in ((minus, minus, -1.0), (ir, minus, 1 / 127), (ir, noise, 1 / 127)):
+        out = torch.ops.amoe.cvmm_quantized(x, s.sel_index, s.sel, pr["keys"], ir_t, inp_res, torch.float32,
+                                            s.out_index, minus, noise_t)
+        assert out.shape == (8, 12, 2, 40)
+        want = O.cvmm_fwd(util.np32(pr["x"]), want_sel.in_index, want_sel.sel_sorted, util.np32(pr["keys"]),
+                          inp_res=inp_res, ir=None if ir_t is minus else util.np32(ir).reshape(-1, 1),
+                          out_index=want_sel.perm,
+                          noise=None if noise_t is minus else util.np32(noise).reshape(1, -1, 40))
+        assert util.rel_err(util.np32(out).reshape(-1, 40), want) < 1e-5
