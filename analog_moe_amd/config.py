@@ -15,6 +15,8 @@ from enum import Enum
 
 class WeightModifierType(Enum):
     NONE = "None"
+    COPY = "Copy"                       # the two AIHWKIT-only members (moe_layer_aihwkit.py:166-170)
+    MULT_NORMAL = "MultNormal"
     DISCRETIZE = "Discretize"
     DISCRETIZE_PER_CHANNEL = "DiscretizePerChannel"
     ADD_NORMAL = "AddNormal"
@@ -25,8 +27,18 @@ class WeightModifierType(Enum):
 
 class WeightClipType(Enum):
     NONE = "None"
+    FIXED_VALUE = "FixedValue"          # AIHWKIT flavour (moe_layer_aihwkit.py:324-340)
+    AVERAGE_CHANNEL_MAX = "AverageChannelMax"
     LAYER_GAUSSIAN = "LayerGaussian"
     LAYER_GAUSSIAN_PER_CHANNEL = "LayerGaussianPerChannel"
+
+
+class WeightRemapType(Enum):
+    """``rpu_config.remap.type`` of the AIHWKIT flavour: which max |W| the analog tile is assumed to be
+    normalised by (moe_layer_aihwkit.py:172-182, 264-279)."""
+    NONE = "None"
+    LAYERWISE_SYMMETRIC = "LayerwiseSymmetric"
+    CHANNELWISE_SYMMETRIC = "ChannelwiseSymmetric"
 
 
 class NoiseManagementType(Enum):
@@ -85,6 +97,7 @@ class WeightModifierParameter:
     res: float = 2 ** 8 - 2
     std_dev: float = 0.0
     enable_during_test: bool = False
+    per_batch_sample: bool = False
 
 
 @dataclass
@@ -95,12 +108,24 @@ class WeightClipParameter:
 
 
 @dataclass
+class WeightRemapParameter:
+    type: WeightRemapType = WeightRemapType.LAYERWISE_SYMMETRIC
+
+
+@dataclass
 class TorchInferenceRPUConfig:
     forward: IOParameters = field(default_factory=IOParameters)
     pre_post: PrePostProcessing = field(default_factory=PrePostProcessing)
     mapping: MappingParameter = field(default_factory=MappingParameter)
     modifier: WeightModifierParameter = field(default_factory=WeightModifierParameter)
     clip: WeightClipParameter = field(default_factory=WeightClipParameter)
+
+
+@dataclass
+class AIHWKITTorchInferenceRPUConfig(TorchInferenceRPUConfig):
+    """The attributes the AIHWKIT flavour reads on top (moe_layer_aihwkit.py:47-61, 243-279)."""
+    forward: AIHWKITIOParameters = field(default_factory=AIHWKITIOParameters)
+    remap: WeightRemapParameter = field(default_factory=WeightRemapParameter)
 
 
 def kernel_inp_res(res: float) -> float:

@@ -24,7 +24,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from .config import (TorchInferenceRPUConfig, WeightClipType, WeightModifierType, enum_name, kernel_inp_res)
+from .config import (AIHWKITTorchInferenceRPUConfig, TorchInferenceRPUConfig, enum_name, kernel_inp_res)
 from .cvmm import CVMM, AnalogExt, CVMMSel, cvmm_prepare_sel2, cvmm_std
 from . import library  # noqa: F401  (registers the amoe:: operators)
 from .ffn import FFNConfig, moe_ffn
@@ -253,6 +253,24 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         if o_bias is not None and self.o_bias is not None:
             self.o_bias.data = o_bias.detach().clone()
 
+    # -- what differs between the two flavours of the reference -------------------------------------------
+    def _io_perfect(self) -> bool:
+        """True switches the DAC, the ADC and the output noise off (only the AIHWKIT flavour can)."""
+        return False
+
+    def _noise_per_channel(self) -> bool:
+        return bool(getattr(self.rpu_config.forward, "out_noise_per_channel", False))
+
+    def _modifier_on(self) -> bool:
+        return enum_name(self.rpu_config.modifier.type) != "NONE"
+
+    def _modified(self, weights: Tensor) -> Tensor:
+        return self.modify_weight(weights.clone(), self.rpu_config.modifier)
+
+    def _row_abs_max_on(self) -> bool:
+        """Whether CVMM will scale every input row by its abs-max (cvmm.py:727-739)."""
+        return self.input_range is None
+
     # -- weight modifier / clipping (moe_layer_aihwkit_lightning.py:313-382, 509-543) -----------------
     @staticmethod
     def modify_weight(inp_weight: Tensor, modifier) -> Tensor:
@@ -357,15 +375,16 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             if ir.dim() == 2:
                 ir = ir[:, :nt]
             bir = ir[sel_indices.sel]                                   # [..., k(, n_tiles)]
-        inp_res = kernel_inp_res(fwd.inp_res)
+        perfect = self._io_perfect()
+        inp_res = -1.0 if perfect else kernel_inp_res(fwd.inp_res)
         modified = weights
-        if (self.training or self.rpu_config.modifier.enable_during_test) and \
-                enum_name(self.rpu_config.modifier.type) != "NONE":
-            modified = self.modify_weight(weights.clone(), self.rpu_config.modifier)
-        ext = AnalogExt(offsets=sel_indices.offsets, bounds=bounds, out_bound=float(getattr(fwd, "out_bound", -1)),
-                        out_res=float(getattr(fwd, "out_res", -1)))
-        per_channel = bool(getattr(fwd, "out_noise_per_channel", False))
-        noisy = self.training and fwd.out_noise > 0
+        if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
+            modified = self._modified(weights)
+        ext = AnalogExt(offsets=sel_indices.offsets, bounds=bounds,
+                        out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
+                        out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
+        per_channel = self._noise_per_channel()
+        noisy = self.training and fwd.out_noise > 0 and not perfect
         if ext.out_bound > 0 or noisy:
             ext.wmax = torch.ops.amoe.weight_abs_max(weights.detach(), per_channel)
         out_noise = None
@@ -385,7 +404,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     # -- fused path ---------------------------------------------------------------------------------------
     def _fusable(self) -> bool:
         return (self.activation is F.relu and self.bias is None and self.dropout == 0 and
-                self.input_range is not None and enum_name(self.rpu_config.modifier.type) == "NONE" and
+                self.input_range is not None and not self._row_abs_max_on() and not self._modifier_on() and
                 not (self.training and self._init_from_data_pending()))
 
     def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
@@ -393,12 +412,15 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             return super().forward_selected(x, sel_val, sel_idx)
         fwd = self.rpu_config.forward
         irp = self.rpu_config.pre_post.input_range
-        noisy = self.training and fwd.out_noise > 0
-        cfg = FFNConfig(inp_res=kernel_inp_res(fwd.inp_res), bounds_up=self.bounds_up, bounds_down=self.bounds_down,
-                        out_bound=float(getattr(fwd, "out_bound", -1)), out_res=float(getattr(fwd, "out_res", -1)),
+        perfect = self._io_perfect()
+        noisy = self.training and fwd.out_noise > 0 and not perfect
+        cfg = FFNConfig(inp_res=-1.0 if perfect else kernel_inp_res(fwd.inp_res), bounds_up=self.bounds_up,
+                        bounds_down=self.bounds_down,
+                        out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
+                        out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)),
                         noise_std=float(fwd.out_noise) if noisy else 0.0, noise_seed=self._noise_seed() if noisy else 0,
                         noise_seed_dev=self.noise_counter if noisy else None,
-                        noise_per_channel=bool(getattr(fwd, "out_noise_per_channel", False)),
+                        noise_per_channel=self._noise_per_channel(),
                         gradient_relative=getattr(irp, "gradient_relative", True),
                         gradient_scale=getattr(irp, "gradient_scale", 1.0), decay=irp.decay,
                         input_min_percentage=irp.input_min_percentage)
@@ -438,6 +460,142 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         self._init_done = False
 
 
-# Names under which the reference exports its two flavours (analog_moe/__init__.py).
+class AnalogSigmaMoELayerAIHWKIT(AnalogSigmaMoELayer):
+    """The reference's second flavour (analog_moe/moe_layer_aihwkit.py:29-436) on the same kernels.  What it
+    does differently from the lightning flavour:
+
+    * ``forward.is_perfect`` switches quantisation and output noise off (:243-258);
+    * the row abs-max scaling follows ``forward.noise_management`` instead of the input range
+      (cvmm.py:735-739), and the bound management must be off (:59-61);
+    * the max |W| behind the output noise and the weight modifier follows ``remap.type`` (:172-182, 264-279);
+    * the weight modifier knows ADD_NORMAL only (:144-196), the clip FIXED_VALUE and LAYER_GAUSSIAN
+      (:313-340);
+    * the configuration travels in the state dict under ``analog_tile_state`` (:372-415).
+
+    AIHWKIT's tile objects (``AnalogContext``, the analog optimizer hooks) are third-party and not part of
+    this package; the K-tile split and the ADC, which the reference asserts off (:50-58), stay available."""
+
+    def __init__(self, rpu_config=None, *args, **kwargs):
+        rpu_config = AIHWKITTorchInferenceRPUConfig() if rpu_config is None else rpu_config
+        fwd = rpu_config.forward
+        if not hasattr(fwd, "is_perfect"):
+            raise MoEConifgError("the AIHWKIT flavour needs an rpu_config whose forward has is_perfect "
+                                 "(an aihwkit TorchInferenceRPUConfig or AIHWKITTorchInferenceRPUConfig)")
+        assert getattr(fwd, "inp_bound", 1.0) in [-1, 1.0], "inp_bound must be 1.0 or off (=-1)"
+        assert enum_name(getattr(fwd, "bound_management", "NONE")) == "NONE", "bound_management must be NONE"
+        super().__init__(rpu_config, *args, **kwargs)
+
+    # -- flavour hooks ---------------------------------------------------------------------------------------
+    def _remap(self) -> str:
+        remap = getattr(self.rpu_config, "remap", None)
+        return "NONE" if remap is None else enum_name(remap.type)
+
+    def _io_perfect(self) -> bool:
+        return bool(self.rpu_config.forward.is_perfect)
+
+    def _noise_per_channel(self) -> bool:
+        kind = self._remap()                                  # moe_layer_aihwkit.py:264-279
+        if kind in ("CHANNELWISE_SYMMETRIC", "NONE"):
+            return True
+        if kind == "LAYERWISE_SYMMETRIC":
+            return False
+        raise MoEConifgError(f"Weight remap type {self.rpu_config.remap.type} not supported")
+
+    def _modifier_on(self) -> bool:
+        return enum_name(self.rpu_config.modifier.type) not in ("NONE", "COPY")
+
+    def _modified(self, weights: Tensor) -> Tensor:
+        return self.modify_weight(weights, self.rpu_config.modifier, self.rpu_config.remap.type)
+
+    def _row_abs_max_on(self) -> bool:
+        fwd = self.rpu_config.forward
+        return not fwd.is_perfect and enum_name(fwd.noise_management) == "ABS_MAX"
+
+    @staticmethod
+    def modify_weight(inp_weight: Tensor, modifier, remap_type=None) -> Tensor:
+        """moe_layer_aihwkit.py:144-196."""
+        if getattr(modifier, "per_batch_sample", False):
+            raise MoEConifgError("per_batch_sample not implemented")
+        kind = enum_name(modifier.type)
+        if kind in ("NONE", "COPY"):
+            return inp_weight
+        if kind == "MULT_NORMAL":
+            raise MoEConifgError("MULT_NORMAL not implemented")
+        remap = enum_name(remap_type)
+        if remap == "CHANNELWISE_SYMMETRIC":
+            wmax = inp_weight.abs().amax(1).unsqueeze(1)                        # [E, 1, N]
+        elif remap == "LAYERWISE_SYMMETRIC":
+            wmax = inp_weight.reshape(inp_weight.size(0), -1).abs().amax(-1).view(-1, 1, 1)
+        else:
+            raise MoEConifgError(f"Weight remap type {remap_type} not supported")
+        if kind == "DISCRETIZE":
+            raise MoEConifgError("DISCRETIZE not implemented")
+        if kind != "ADD_NORMAL":
+            raise MoEConifgError(f"Weight modifier {modifier} not supported")
+        with torch.no_grad():
+            noise = modifier.std_dev * wmax * torch.randn(inp_weight.shape, device=inp_weight.device)
+        return inp_weight.clone() + noise.to(inp_weight.dtype)
+
+    def post_update_step(self) -> None:
+        if hasattr(self.rpu_config, "clip") and enum_name(self.rpu_config.clip.type) != "NONE":
+            self.clip_weights(self.rpu_config.clip)
+
+    @torch.no_grad()
+    def clip_weights(self, clip=None) -> None:
+        """moe_layer_aihwkit.py:313-340."""
+        clip = self.rpu_config.clip if clip is None else clip
+        kind = enum_name(clip.type)
+        if kind == "FIXED_VALUE":
+            for w in (self.keys, self.values):
+                w.data = torch.clamp(w, -clip.fixed_value, clip.fixed_value)
+        elif kind == "LAYER_GAUSSIAN":
+            for w in (self.keys, self.values):
+                alpha = w.std((1, 2), keepdim=True) * clip.sigma
+                if clip.fixed_value > 0:
+                    alpha = alpha.clamp(max=clip.fixed_value)
+                w.data = torch.minimum(torch.maximum(w.data, -alpha), alpha)
+        elif kind == "AVERAGE_CHANNEL_MAX":
+            raise NotImplementedError("AVERAGE_CHANNEL_MAX not implemented")
+        else:
+            raise MoEConifgError(f"Unknown clip type {clip.type}")
+
+    def get_dtype(self) -> torch.dtype:
+        return self.keys.dtype
+
+    # -- checkpointing (moe_layer_aihwkit.py:372-436) --------------------------------------------------------------
+    def load_state_dict(self, state_dict, strict: bool = True, load_rpu_config: Optional[bool] = None,
+                        strict_rpu_config_check: Optional[bool] = None, **kwargs):
+        state_dict = state_dict.copy()
+        analog_tile_state = state_dict.pop("analog_tile_state", None)
+        if analog_tile_state is not None:
+            if strict_rpu_config_check:
+                ok, msg = self.compatible_with(analog_tile_state["rpu_config"])
+                if not ok:
+                    raise MoEConifgError(msg)
+            if load_rpu_config or load_rpu_config is None:
+                self.rpu_config = analog_tile_state["rpu_config"]
+        self._init_done = False
+        return nn.Module.load_state_dict(self, state_dict, strict, **kwargs)
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        nn.Module._save_to_state_dict(self, destination, prefix, keep_vars)
+        destination[prefix + "analog_tile_state"] = {"rpu_config": self.rpu_config}
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        analog_tile_state = state_dict.pop(prefix + "analog_tile_state", None)
+        if analog_tile_state is not None:
+            self.rpu_config = analog_tile_state["rpu_config"]
+        nn.Module._load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys,
+                                        unexpected_keys, error_msgs)
+        self._init_done = False
+
+    def compatible_with(self, rpu_config) -> Tuple[bool, Optional[str]]:
+        if not isinstance(self.rpu_config, type(rpu_config)) and not isinstance(rpu_config, type(self.rpu_config)):
+            return False, ("RPU config mismatch: Cannot replace "
+                           f"{rpu_config.__class__.__name__} with {self.rpu_config.__class__.__name__}")
+        return True, None
+
+
+# Name under which the reference exports its lightning flavour (analog_moe/__init__.py).
 AnalogSigmaMoELayerAIHWKITLightning = AnalogSigmaMoELayer
-AnalogSigmaMoELayerAIHWKIT = AnalogSigmaMoELayer

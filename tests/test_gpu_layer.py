@@ -278,3 +278,85 @@ def test_reference_operator_matches_oracle():
                           out_index=want_sel.perm,
                           noise=None if noise_t is minus else util.np32(noise).reshape(1, -1, 40))
         assert util.rel_err(util.np32(out).reshape(-1, 40), want) < 1e-5
+
+
+def _aihwkit_layer(cfgmod, d=128, E=4, F=64, k=2, ir=True, **fw):
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayerAIHWKIT
+    r = cfgmod.AIHWKITTorchInferenceRPUConfig()
+    r.forward.inp_res = 2 ** 8 - 2
+    for name, v in fw.items():
+        setattr(r.forward, name, v)
+    r.pre_post.input_range.enable = ir
+    r.pre_post.input_range.init_value = 2.0
+    torch.manual_seed(0)
+    return AnalogSigmaMoELayerAIHWKIT(r, d_model=d, n_experts=E, expert_size=F, k=k).cuda()
+
+
+def test_aihwkit_flavour_perfect_io_equals_the_digital_layer():
+    """forward.is_perfect (moe_layer_aihwkit.py:243-258): no quantisation, no noise, no abs-max scaling --
+    with the input ranges off this is the digital SigmaMoE layer, forward and backward."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayerAIHWKIT
+    layer = _aihwkit_layer(cfgmod, ir=False, is_perfect=True, out_noise=0.1)
+    layer.train()
+    dig = AnalogSigmaMoELayerAIHWKIT.to_digital(layer)
+    x = torch.randn(5, 9, 128, device="cuda")
+    outs = []
+    for m in (layer, dig):
+        xi = x.clone().requires_grad_()
+        y, reg = m(xi)
+        (y.square().sum() + reg).backward()
+        outs.append((y, xi.grad, m.keys.grad, m.values.grad, m.expert_sel.weight.grad))
+    for a, b in zip(*outs):
+        assert util.rel_err(util.np32(a), util.np32(b)) < 1e-5
+
+
+def test_aihwkit_flavour_abs_max_follows_noise_management():
+    """cvmm.py:735-739: ABS_MAX scales every input row by its abs-max (and is scale-equivariant with the
+    ranges off); it gives what the lightning flavour gives with its ranges disabled (cvmm.py:729-733)."""
+    from analog_moe_amd import config as cfgmod
+    a_layer = _aihwkit_layer(cfgmod, ir=False, noise_management=cfgmod.NoiseManagementType.ABS_MAX)
+    l_layer = _layer(cfgmod, {}, ir=False)
+    l_layer.load_state_dict(a_layer.state_dict(), strict=False)
+    x = torch.randn(6, 7, 128, device="cuda")
+    sel_val, sel_idx, _ = a_layer.select(x)
+    a = a_layer.forward_selected(x, sel_val, sel_idx)
+    assert torch.allclose(4 * a, a_layer.forward_selected(4 * x, sel_val, sel_idx), rtol=1e-5, atol=1e-6)
+    assert torch.equal(a, l_layer.forward_selected(x, sel_val, sel_idx))
+    # with the ranges on both scalings apply: clamp(x, +-ir) / ir, then the division by the abs-max of the RAW
+    # row (cvmm.py:737 takes it from x itself)
+    both = _aihwkit_layer(cfgmod, ir=True, noise_management=cfgmod.NoiseManagementType.ABS_MAX)
+    assert both._row_abs_max_on() and not both._fusable()
+    s = O.prepare_sel(sel_idx.reshape(-1, 2).cpu().numpy(), 4, 2)
+    x2 = util.np32(x.reshape(-1, 128))
+    am = np.abs(x2).max(-1)
+    want = O.cvmm_fwd(x2, s.in_index, s.sel_sorted, util.np32(both.keys), inp_res=1 / 127,
+                      ir=np.full((s.sel_sorted.size, 1), 2.0, np.float32), out_index=s.perm, abs_max=am)
+    from analog_moe_amd.cvmm import cvmm_prepare_sel2
+    got = both.cvmm_wrapper(x, cvmm_prepare_sel2(sel_idx, 4), both.keys)
+    assert util.rel_err(util.np32(got).reshape(-1, 64), want) < 1e-5
+
+
+@pytest.mark.parametrize("remap", ["LAYERWISE_SYMMETRIC", "CHANNELWISE_SYMMETRIC"])
+def test_aihwkit_flavour_noise_scale_follows_remap_type(remap):
+    """moe_layer_aihwkit.py:264-279: the output noise is out_noise x max |W| per expert (layerwise) or per
+    output channel (channelwise)."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.cvmm import cvmm_prepare_sel2
+    layer = _aihwkit_layer(cfgmod, d=64, E=2, F=64, k=1, out_noise=0.1, inp_res=-1)
+    layer.rpu_config.remap.type = cfgmod.WeightRemapType[remap]
+    with torch.no_grad():
+        layer.input_range.fill_(1.0)
+        layer.keys[:, :, :8] *= 8.0                      # eight loud output channels per expert
+    x = torch.randn(4096, 1, 64, device="cuda").clamp(-0.9, 0.9)
+    sel = cvmm_prepare_sel2(torch.randint(0, 2, (4096, 1, 1), device="cuda"), 2)
+    layer.eval()
+    clean = layer.cvmm_wrapper(x, sel, layer.keys)
+    layer.train()
+    noise = (layer.cvmm_wrapper(x, sel, layer.keys) - clean).reshape(4096, 64)
+    for e in range(2):
+        rows = sel.raw_sel.reshape(-1) == e
+        spread = noise[rows].std(0)
+        w = layer.keys[e].detach().abs()
+        want = 0.1 * (w.amax(0) if remap == "CHANNELWISE_SYMMETRIC" else w.max().expand(64))
+        assert torch.allclose(spread, want, rtol=0.15)

@@ -9,7 +9,8 @@ import pytest
 import torch
 
 from analog_moe_amd import _abi, config as cfg
-from analog_moe_amd.moe_layer import AnalogSigmaMoELayer, MoEConifgError, SigmaMoELayer, tile_bounds
+from analog_moe_amd.moe_layer import (AnalogSigmaMoELayer, AnalogSigmaMoELayerAIHWKIT, MoEConifgError, SigmaMoELayer,
+                                      tile_bounds)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -93,6 +94,101 @@ def test_inp_res_mapping_and_weight_modifier():
     before = layer.keys.data.abs().max().item()
     layer.post_update_step()
     assert layer.keys.data.abs().max().item() < before
+
+
+def _aihwkit_rpu(**fw):
+    r = cfg.AIHWKITTorchInferenceRPUConfig()
+    r.forward.inp_res = 2 ** 8 - 2
+    for k, v in fw.items():
+        setattr(r.forward, k, v)
+    r.pre_post.input_range.enable = True
+    return r
+
+
+def test_aihwkit_flavour_configuration_rules():
+    """moe_layer_aihwkit.py:47-61 (constructor checks), :243-258 (is_perfect), :264-279 (remap type picks the
+    max |W| behind the noise), cvmm.py:735-739 (abs-max follows the noise management)."""
+    kw = dict(d_model=16, n_experts=3, expert_size=8, k=1)
+    layer = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), **kw)
+    assert isinstance(layer.rpu_config, cfg.AIHWKITTorchInferenceRPUConfig) and layer.input_range.shape == (2, 3)
+    assert not layer._io_perfect() and not layer._row_abs_max_on() and layer._fusable()
+    assert layer._noise_per_channel() is False                               # LAYERWISE_SYMMETRIC
+    layer.rpu_config.remap.type = cfg.WeightRemapType.CHANNELWISE_SYMMETRIC
+    assert layer._noise_per_channel() is True
+    layer.rpu_config.remap.type = cfg.WeightRemapType.NONE
+    assert layer._noise_per_channel() is True
+    layer.rpu_config.forward.noise_management = cfg.NoiseManagementType.ABS_MAX
+    assert layer._row_abs_max_on() and not layer._fusable()
+    layer.rpu_config.forward.is_perfect = True
+    assert layer._io_perfect() and not layer._row_abs_max_on()
+    assert AnalogSigmaMoELayerAIHWKIT(None, **kw).input_range is None          # default config: ranges off
+    with pytest.raises(AssertionError):
+        AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(inp_bound=2.0), **kw)
+    with pytest.raises(AssertionError):
+        AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(bound_management="Iterative"), **kw)
+    with pytest.raises(MoEConifgError):
+        AnalogSigmaMoELayerAIHWKIT(_rpu(), **kw)                             # a lightning config: no is_perfect
+
+
+def test_aihwkit_flavour_modifier_and_clip():
+    """moe_layer_aihwkit.py:144-196 and :313-340."""
+    torch.manual_seed(0)
+    w = torch.randn(3, 64, 40)
+    w[:, :, 0] *= 10
+    M, R = cfg.WeightModifierParameter, cfg.WeightRemapType
+    mod = AnalogSigmaMoELayerAIHWKIT.modify_weight
+    assert mod(w, M(type=cfg.WeightModifierType.NONE), R.LAYERWISE_SYMMETRIC) is w
+    assert mod(w, M(type=cfg.WeightModifierType.COPY), R.LAYERWISE_SYMMETRIC) is w
+    add = M(type=cfg.WeightModifierType.ADD_NORMAL, std_dev=0.1)
+    d_layer = mod(w, add, R.LAYERWISE_SYMMETRIC) - w
+    d_chan = mod(w, add, R.CHANNELWISE_SYMMETRIC) - w
+    wmax_layer = w.reshape(3, -1).abs().amax(-1)
+    assert torch.allclose(d_layer.reshape(3, -1).std(-1), 0.1 * wmax_layer, rtol=0.1)
+    assert torch.allclose(d_chan.std(1), 0.1 * w.abs().amax(1), rtol=0.35)   # 64 samples per channel
+    assert d_chan[:, :, 0].std() > 3 * d_chan[:, :, 1:].std()
+    for bad in (M(type=cfg.WeightModifierType.MULT_NORMAL), M(type=cfg.WeightModifierType.DISCRETIZE),
+                M(type=cfg.WeightModifierType.ADD_NORMAL, per_batch_sample=True)):
+        with pytest.raises(MoEConifgError):
+            mod(w, bad, R.LAYERWISE_SYMMETRIC)
+    with pytest.raises(MoEConifgError):
+        mod(w, add, R.NONE)
+    layer = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), d_model=8, n_experts=3, expert_size=5, k=1)
+    layer.rpu_config.clip = cfg.WeightClipParameter(type=cfg.WeightClipType.FIXED_VALUE, fixed_value=0.05)
+    layer.post_update_step()
+    assert layer.keys.data.abs().max().item() <= 0.05 + 1e-7 and layer.values.data.abs().max().item() <= 0.05 + 1e-7
+    layer.reset_parameters()
+    std = layer.keys.data.std((1, 2), keepdim=True)
+    layer.clip_weights(cfg.WeightClipParameter(type=cfg.WeightClipType.LAYER_GAUSSIAN, sigma=1.0))
+    assert bool((layer.keys.data.abs() <= std * (1 + 1e-6)).all())
+    with pytest.raises(NotImplementedError):
+        layer.clip_weights(cfg.WeightClipParameter(type=cfg.WeightClipType.AVERAGE_CHANNEL_MAX))
+
+
+def test_aihwkit_flavour_state_dict_carries_the_config():
+    """moe_layer_aihwkit.py:372-436: ``analog_tile_state`` entry, load_rpu_config, compatibility check."""
+    kw = dict(d_model=8, n_experts=3, expert_size=4, k=1)
+    layer = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(out_noise=0.07), **kw)
+    sd = layer.state_dict()
+    assert sd["analog_tile_state"]["rpu_config"] is layer.rpu_config
+    assert set(sd) == {"keys", "values", "expert_sel.weight", "input_range", "input_range_update_idx",
+                       "analog_tile_state"}
+    other = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), **kw)
+    other.load_state_dict(sd, load_rpu_config=True, strict_rpu_config_check=True)
+    assert other.rpu_config.forward.out_noise == 0.07 and torch.equal(other.keys, layer.keys)
+    assert "analog_tile_state" in sd                                         # the caller's dict is left alone
+    keep = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), **kw)
+    keep.load_state_dict(sd, load_rpu_config=False)
+    assert keep.rpu_config.forward.out_noise == 0.0
+    assert layer.compatible_with(cfg.AIHWKITTorchInferenceRPUConfig()) == (True, None)
+    ok, msg = layer.compatible_with(object())
+    assert ok                                                                # every class derives from object
+    ok, msg = layer.compatible_with(3)
+    assert not ok and "RPU config mismatch" in msg
+    holder = torch.nn.Sequential(AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(out_noise=0.02), **kw))
+    twin = torch.nn.Sequential(AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), **kw))
+    twin.load_state_dict(holder.state_dict())
+    assert twin[0].rpu_config.forward.out_noise == 0.02
+    assert layer.get_dtype() == torch.float32
 
 
 def test_library_exports_every_declared_symbol():
