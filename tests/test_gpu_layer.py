@@ -360,3 +360,43 @@ def test_aihwkit_flavour_noise_scale_follows_remap_type(remap):
         w = layer.keys[e].detach().abs()
         want = 0.1 * (w.amax(0) if remap == "CHANNELWISE_SYMMETRIC" else w.max().expand(64))
         assert torch.allclose(spread, want, rtol=0.15)
+
+
+@pytest.mark.parametrize("use_abs_max", [True, False])
+def test_aihwkit_flavour_ir_gradient_recipe(use_abs_max):
+    """The recipe of the reference's tests/test_moe_layer_aihwkit.py:180-306 (d_model 128, 4 experts of 64,
+    k = 2, 10 x 10 tokens, no quantisation, loss = sum; tolerances 1e-4, input gradient 1e-3): with ABS_MAX
+    and no input ranges the scaling cancels and the layer equals the digital one; otherwise the input ranges
+    are 1..4 per expert and outputs and all gradients, the ranges' included, follow the closed forms."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayerAIHWKIT
+    nm = cfgmod.NoiseManagementType.ABS_MAX if use_abs_max else cfgmod.NoiseManagementType.NONE
+    layer = _aihwkit_layer(cfgmod, ir=not use_abs_max, inp_res=-1, noise_management=nm)
+    layer.train()
+    x = torch.randn(10, 10, 128, device="cuda", requires_grad=True)
+    if use_abs_max:
+        dig = AnalogSigmaMoELayerAIHWKIT.to_digital(layer)
+        x2 = x.detach().clone().requires_grad_()
+        ya, _ = layer(x)
+        yd, _ = dig(x2)
+        ya.sum().backward()
+        yd.sum().backward()
+        assert torch.allclose(ya, yd, atol=1e-4)
+        assert torch.allclose(layer.keys.grad, dig.keys.grad, atol=1e-4)
+        assert torch.allclose(layer.values.grad, dig.values.grad, atol=1e-4)
+        assert torch.allclose(x.grad, x2.grad, atol=1e-3)
+        return
+    with torch.no_grad():
+        layer.input_range.copy_(torch.tensor([[1.0, 2.0, 3.0, 4.0]] * 2))
+    sel_val, sel_idx, _ = layer.select(x.detach())
+    sel_val = sel_val.detach().requires_grad_()
+    y = layer.forward_selected(x, sel_val, sel_idx)
+    y.sum().backward()
+    want = _oracle_for(layer, x, sel_val, sel_idx, torch.ones_like(y), inp_res=-1, decay=0.0,
+                       input_min_percentage=0.95)
+    assert np.allclose(util.np32(y).reshape(100, 128), want.y, atol=1e-4)
+    assert np.allclose(util.np32(layer.keys.grad), want.grad_keys, atol=1e-4)
+    assert np.allclose(util.np32(layer.values.grad), want.grad_values, atol=1e-4)
+    assert np.allclose(util.np32(x.grad).reshape(100, 128), want.grad_x, atol=1e-3)
+    assert np.allclose(util.np32(layer.input_range.grad), want.grad_ir.reshape(2, 4), atol=1e-4)
+    assert np.abs(want.grad_ir).max() > 0                       # ranges 1 and 2 do clip N(0,1) inputs
