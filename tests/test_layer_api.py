@@ -206,3 +206,78 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(raw, name), name
     assert raw.amoe_version() == 100
     assert ctypes.sizeof(_abi.FwdArgs) % 8 == 0
+
+
+def test_library_rejects_bad_arguments_on_the_host():
+    """Arguments are validated before anything is launched, so the documented codes of include/amoe.h come
+    back from the built library without a GPU: NULL / size / shape / alignment / workspace errors."""
+    path = os.path.join(ROOT, "analog_moe_amd", "csrc", "libamoe.so")
+    if not os.path.exists(path):
+        pytest.skip("libamoe.so has not been built")
+    lib = _abi.bind(path)
+    EINVAL, ENULL, ESHAPE, EALIGN, EWORKSPACE, EUNSUPPORTED = -1, -2, -3, -4, -5, -6
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)                                   # host memory: only ever looked at as an address
+    assert lib.amoe_cvmm_fwd(None, None) == ENULL
+    assert lib.amoe_cvmm_bwd_w(None, None) == ENULL
+    assert lib.amoe_cvmm_bwd_x(None, None) == ENULL
+    # selection
+    assert lib.amoe_prepare_sel(p, 0, -1, 4, 2, p, p, p, p, None, p, 4096, None) == EINVAL
+    assert lib.amoe_prepare_sel(p, 0, 16, 0, 2, p, p, p, p, None, p, 4096, None) == EINVAL
+    assert lib.amoe_prepare_sel(p, 0, 16, 4096, 2, p, p, p, p, None, p, 4096, None) == EUNSUPPORTED
+    assert lib.amoe_prepare_sel(None, 0, 16, 4, 2, p, p, p, p, None, p, 4096, None) == ENULL
+    assert lib.amoe_prepare_sel(p, 0, 16, 4, 2, p + 2, p, p, p, None, p, 4096, None) == EALIGN
+    assert lib.amoe_prepare_sel(p, 0, 16, 4, 2, p, p, p, p, None, p, 0, None) == EWORKSPACE
+    assert lib.amoe_offsets_from_sorted(None, 8, 4, p, None) == ENULL
+    # forward
+    def fwd(**kw):
+        a = _abi.FwdArgs(dtype=_abi.AMOE_F32, M=8, N=16, K=32, E=2, n_in_rows=8, n_out_rows=8, x=p, ldx=32, w=p,
+                         w_stride_e=512, w_stride_k=16, w_stride_n=1, out=p, ldo=16, sel_sorted=p, offsets=p,
+                         in_index=p, inp_res=-1.0, n_tiles=1, out_bound=-1.0, out_res=-1.0)
+        a.tile_bounds[0], a.tile_bounds[1] = 0, 32
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert lib.amoe_cvmm_fwd(fwd(dtype=7), None) == EINVAL
+    assert lib.amoe_cvmm_fwd(fwd(K=0), None) == EINVAL
+    assert lib.amoe_cvmm_fwd(fwd(x=None), None) == ENULL
+    assert lib.amoe_cvmm_fwd(fwd(ldx=16), None) == ESHAPE
+    assert lib.amoe_cvmm_fwd(fwd(w_stride_k=3, w_stride_n=5), None) == EUNSUPPORTED
+    assert lib.amoe_cvmm_fwd(fwd(n_tiles=0), None) == EINVAL
+    assert lib.amoe_cvmm_fwd(fwd(n_tiles=_abi.AMOE_MAX_TILES + 1), None) == EINVAL
+    bad = fwd()
+    bad.tile_bounds[1] = 31                                     # the last bound must be K
+    assert lib.amoe_cvmm_fwd(bad, None) == ESHAPE
+    assert lib.amoe_cvmm_fwd(fwd(out_bound=12.0), None) == ESHAPE          # ADC without max |W|
+    assert lib.amoe_cvmm_fwd(fwd(noise_std=0.1), None) == ESHAPE           # generated noise without max |W|
+    assert lib.amoe_cvmm_fwd(fwd(xq_out=p), None) == EINVAL                # second output without its range
+    assert lib.amoe_cvmm_fwd(fwd(x=p + 2), None) == EALIGN
+    # gradients
+    def bwd_w(**kw):
+        a = _abi.BwdWArgs(dtype=_abi.AMOE_F32, M=8, N=16, K=32, E=2, x=p, ldx=32, g=p, ldg=16, grad_w=p, offsets=p,
+                          in_index=p, n_x_rows=8, n_g_rows=8, n_tiles=1)
+        a.tile_bounds[0], a.tile_bounds[1] = 0, 32
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert lib.amoe_cvmm_bwd_w(bwd_w(dtype=9), None) == EINVAL
+    assert lib.amoe_cvmm_bwd_w(bwd_w(grad_w=None), None) == ENULL
+    assert lib.amoe_cvmm_bwd_w(bwd_w(ldg=8), None) == ESHAPE
+    def bwd_x(**kw):
+        a = _abi.BwdXArgs(dtype=_abi.AMOE_F32, M=8, N=16, K=32, E=2, g=p, ldg=16, n_g_rows=8, w=p, w_stride_e=512,
+                          w_stride_k=16, grad_x_full=p, ldo=32, offsets=p, g_index=p, out_index=p, n_tiles=1)
+        a.tile_bounds[0], a.tile_bounds[1] = 0, 32
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert lib.amoe_cvmm_bwd_x(bwd_x(E=0), None) == EINVAL
+    assert lib.amoe_cvmm_bwd_x(bwd_x(g_index=None), None) == ENULL
+    assert lib.amoe_cvmm_bwd_x(bwd_x(relu_mask=1), None) == ENULL          # a mask needs the forward input
+    assert lib.amoe_cvmm_bwd_x(bwd_x(ldo=16), None) == ESHAPE
+    # companions
+    assert lib.amoe_gate_reduce(_abi.AMOE_F32, p, None, p, 4, 2, 8, None) == ENULL
+    assert lib.amoe_gate_grad(5, p, p, p, 4, 2, 8, None) == EINVAL
+    assert lib.amoe_row_abs_max(_abi.AMOE_F32, p, 4, 8, 16, p, None) == EINVAL          # ldx < K
+    assert lib.amoe_weight_abs_max(_abi.AMOE_F32, p, 2, 8, 16, 3, p, None) == EINVAL   # cols is 1 or N
+    for rc in (EINVAL, ENULL, ESHAPE, EALIGN, EWORKSPACE, EUNSUPPORTED):
+        assert len(lib.amoe_strerror(rc)) > 0
