@@ -207,7 +207,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
     const int rt = w / ncb, cb = w - rt * ncb;
     {                                       // this item's row tile: gather pointers, scatter rows
       cur_rt = rt;
-      e = sDesc[it][0]; row0 = sDesc[it][1]; row_end = sDesc[it][2];
+      // (the same for every lane: kept in scalar registers, and so is everything derived from them)
+      e = wave_uniform(sDesc[it][0]); row0 = wave_uniform(sDesc[it][1]); row_end = wave_uniform(sDesc[it][2]);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int r = row0 + (tid >> 3) + 32 * i;
@@ -332,12 +333,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       auto store_step = [&](int buf, Raw (&ra)[4], Raw (&rb)[4]) {   // registers -> LDS stage, DAC stage on the way
         T* __restrict__ dA = sStage + buf * STAGE;
         T* __restrict__ dB = dA + A_ELEMS;
+        if (FWD && dac_ir_quant) {      // the usual input stage: clip, scale, round (one branch for all chunks)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          Raw a = ra[i];
-          if (FWD && dac_ir_quant) {
+          for (int i = 0; i < 4; i++) {
             float v[CH];
-            raw_unpack<T>(a, v);
+            raw_unpack<T>(ra[i], v);
             const float r = a_ir[i], rinv = a_ir_inv[i];
 #pragma unroll
             for (int j = 0; j < CH; j++) {
@@ -345,9 +345,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
               const float c = rintf(div_by(div_by(x, r, rinv), p.inp_res, inv_res));
               v[j] = IS_BF16 ? c : c * p.inp_res;
             }
-            if constexpr (IS_BF16) a = raw_pack_exact_bf16(v);
-            else a = raw_pack<T>(v);
-          } else if (!FAST && FWD && dac) {
+            if constexpr (IS_BF16) ra[i] = raw_pack_exact_bf16(v);
+            else ra[i] = raw_pack<T>(v);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          Raw a = ra[i];
+          if (!FAST && FWD && dac && !dac_ir_quant) {
             float v[CH];
             raw_unpack<T>(a, v);
             bool out_of_range = false;
@@ -462,6 +467,40 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
             for (int b = 0; b < 2; b++) total[a][b] += acc[a][b];
         }
+      } else if (FWD && FAST && codes_mode && gen_noise && adc_quant && col_uniform && has_ir) {
+        // The usual training configuration on edge-free tiles -- DAC codes, noise drawn here, ADC with one
+        // max |W| per expert, input range -- as straight-line code: same operations in the same order as the
+        // general stage below, without a branch around every 4 values.
+        const NoiseKey key = noise_key(seed, t);
+#pragma unroll
+        for (int ti = 0; ti < 2; ti++) {
+          const int rl = wr * 64 + ti * 32 + l32;
+          const int r = row0 + rl;
+          const bool valid = r < row_end;
+          const int orow = valid ? sOrow[rl] : 0;
+          const float ir_r = valid ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + t] : 1.f;
+          const uint32_t row_key = noise_row_key(key, (uint32_t)orow);
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
+              float z[4];
+              noise_pair(key, row_key, (uint32_t)(col >> 1), z[0], z[1]);
+              noise_pair(key, row_key, (uint32_t)(col >> 1) + 1u, z[2], z[3]);
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                float v = acc[fi][ti][4 * q + j] * p.inp_res;
+                v += u_nz * z[j];
+                v = clamp_sym(v, u_bound);
+                v = rintf(v * u_q) * u_qinv;
+                v *= ir_r;
+                if (MODE == MODE_FWD_SPLIT) total[fi][ti][4 * q + j] += v;
+                else acc[fi][ti][4 * q + j] = v;
+              }
+            }
+          }
+        }
       } else if (FWD) {
         const NoiseKey key = noise_key(seed, t);
 #pragma unroll
@@ -549,13 +588,80 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
       // input gradient: clip mask, input-range gradient partial sums, gate
       const T* __restrict__ XF = static_cast<const T*>(p.xf);
       const T* __restrict__ GATE = static_cast<const T*>(p.gate);
+      if (xf_stage) {
+        // Edge-free, mask tile parked in LDS: straight-line code.  A stage that is switched off works with a
+        // neutral constant (infinite range, threshold -inf, gate 1) instead of a branch around every 4 values.
+        T* __restrict__ sXF = sStage + (((p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK) & 1) * STAGE;
+        const float kInf = __builtin_inff();
+        const float relu_thr = p.relu_mask ? 0.f : -kInf;
+#pragma unroll
+        for (int ti = 0; ti < 2; ti++) {
+          const int rl = wr * 64 + ti * 32 + l32;
+          const int r = row0 + rl;
+          const bool valid = r < row_end;
+          const int orow = valid ? sOrow[rl] : 0;
+          const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
+          const float ir_r = (use_ir_bw && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile]
+                                                  : kInf;
+          float part = 0.f;
+          int seen = 0;
+#pragma unroll
+          for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              float xv[4];
+              load4<T>(&sXF[rl * LDO + wc * 64 + fi * 32 + 8 * q + 4 * lh], xv, 4, true);
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                float g = acc[fi][ti][4 * q + j];
+                const float gs = g * gate_r;
+                part += xv[j] >= ir_r ? fminf(gs, 0.f) : 0.f;
+                part -= xv[j] <= -ir_r ? fmaxf(gs, 0.f) : 0.f;
+                const bool not_clip = fabsf(xv[j]) < ir_r;
+                seen += not_clip ? 1 : 0;
+                g = not_clip ? g : 0.f;
+                g = xv[j] > relu_thr ? g : 0.f;
+                acc[fi][ti][4 * q + j] = g * gate_r;
+              }
+            }
+          }
+          cnt += valid ? seen : 0;
+          if (use_ir_bw) {
+            part += wave_shfl_xor(part, 32);
+            if (lh == 0) sRed[wc][rl] = part;
+          }
+        }
+        if (p.xc_out != nullptr) {      // the clipped, gate-scaled input for the weight gradient, in place
+#pragma unroll
+          for (int ti = 0; ti < 2; ti++) {
+            const int rl = wr * 64 + ti * 32 + l32;
+            const int r = row0 + rl;
+            const bool valid = r < row_end;
+            const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + sOrow[rl]) : 1.f;
+            const float ir_r = (use_ir_bw && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile]
+                                                    : kInf;
+#pragma unroll
+            for (int fi = 0; fi < 2; fi++) {
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                T* __restrict__ at = &sXF[rl * LDO + wc * 64 + fi * 32 + 8 * q + 4 * lh];
+                float xv[4];
+                load4<T>(at, xv, 4, true);
+#pragma unroll
+                for (int j = 0; j < 4; j++) xv[j] = clamp_sym(xv[j], ir_r) * gate_r;
+                store4<T>(at, xv, 4, true);
+              }
+            }
+          }
+        }
+      } else if (XF != nullptr || GATE != nullptr) {
 #pragma unroll
       for (int ti = 0; ti < 2; ti++) {
         const int rl = wr * 64 + ti * 32 + l32;
         const int r = row0 + rl;
         const bool valid = r < row_end;
         const int orow = valid ? sOrow[rl] : 0;
-        const int xrow = (valid && XF != nullptr && !xf_stage) ? p.xf_index[r] : 0;
+        const int xrow = (valid && XF != nullptr) ? p.xf_index[r] : 0;
         const float gate_r = (valid && GATE != nullptr) ? Elem<T>::load(GATE + orow) : 1.f;
         const float ir_r = (use_ir_bw && valid) ? p.ir[(int64_t)(p.ir_by_expert ? e : r) * p.ir_cols + colb.tile]
                                                 : 0.f;
@@ -569,20 +675,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
             if (FAST) nv = valid ? 4 : 0;
             float xv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (xf_stage) {
-              const int nst = (p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK;
-              load4<T>(&sStage[(nst & 1) * STAGE + rl * LDO + col - c0], xv, 4, true);
-            } else if (XF != nullptr && nv > 0) {
+            if (XF != nullptr && nv > 0) {
               load4<T>(XF + (int64_t)xrow * p.ldxf + col, xv, nv, FAST || p.xf_vec != 0);
             }
             if (p.xc_out != nullptr) {      // the clipped, gate-scaled input for the weight gradient
               float pc[4];
 #pragma unroll
               for (int j = 0; j < 4; j++) pc[j] = (use_ir_bw ? clamp_sym(xv[j], ir_r) : xv[j]) * gate_r;
-              if (xf_stage) {               // in place: it leaves with the tile below
-                const int nst = (p.kd_bounds[1] - p.kd_bounds[0] + BK - 1) / BK;
-                store4<T>(&sStage[(nst & 1) * STAGE + rl * LDO + col - c0], pc, 4, true);
-              } else if (nv > 0) {
+              if (nv > 0) {
                 store4<T>(static_cast<T*>(p.xc_out) + (int64_t)xrow * p.ldxc + col, pc, nv, p.xc_vec != 0);
               }
             }
@@ -608,6 +708,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           part += wave_shfl_xor(part, 32);
           if (lh == 0) sRed[wc][rl] = part;
         }
+      }
       }
     }
 

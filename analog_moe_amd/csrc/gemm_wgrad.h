@@ -133,7 +133,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   const T* __restrict__ GS = static_cast<const T*>(p.g_scale);
   const bool has_ir = p.ir != nullptr;
   const int chunk = tid % CPR;
-  const float ir_expert = (has_ir && p.ir_by_expert) ? p.ir[(int64_t)e * p.n_tiles + kcol.tile] : 1.f;
+  // (without input ranges the clip below runs against an infinite range: no branch per row group)
+  const float ir_expert = (has_ir && p.ir_by_expert) ? p.ir[(int64_t)e * p.n_tiles + kcol.tile] : __builtin_inff();
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -204,28 +205,23 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   auto store_step = [&](int buf, int mbuf) {  // registers -> LDS, clip / row scaling of x on the way
     T* __restrict__ dX = sX + buf * STAGE;
     T* __restrict__ dG = sG + buf * STAGE;
+    if (has_ir || GS != nullptr) {           // one branch for the whole step; a stage that is off is neutral
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int* m = meta(mbuf, tid / CPR + RPP * i);
+        const float scale = as_f32((uint32_t)m[2]), rng = as_f32((uint32_t)m[3]);
+        float v[CH];
+        raw_unpack<T>(rx[i], v);
+#pragma unroll
+        for (int q = 0; q < CH; q++) v[q] = clamp_sym(v[q], rng) * scale;
+        rx[i] = raw_pack<T>(v);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int j = tid / CPR + RPP * i;
-      Raw x = rx[i];
-      const Raw g = rg[i];
-      if (has_ir || GS != nullptr) {
-        const int* m = meta(mbuf, j);
-        const float scale = as_f32((uint32_t)m[2]), rng = as_f32((uint32_t)m[3]);
-        float v[CH];
-        raw_unpack<T>(x, v);
-        if (has_ir) {
-#pragma unroll
-          for (int q = 0; q < CH; q++) v[q] = clamp_sym(v[q], rng);
-        }
-        if (GS != nullptr) {
-#pragma unroll
-          for (int q = 0; q < CH; q++) v[q] *= scale;
-        }
-        x = raw_pack<T>(v);
-      }
-      *reinterpret_cast<Raw*>(&dX[j * LD + chunk * CH]) = x;
-      *reinterpret_cast<Raw*>(&dG[j * LD + chunk * CH]) = g;
+      *reinterpret_cast<Raw*>(&dX[j * LD + chunk * CH]) = rx[i];
+      *reinterpret_cast<Raw*>(&dG[j * LD + chunk * CH]) = rg[i];
     }
   };
 

@@ -174,11 +174,13 @@ def test_row_chunked_weight_gradient(emu_ops, dtype):
     util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=200)
 
 
-@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
-def test_chained_projections(emu_ops, dtype, D, F):
-    util.check_chained_projections(emu_ops, dtype=dtype, T=60, D=D, F=F)
+@pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 128, 128, 60), (torch.bfloat16, 128, 128, 60),
+                                         (torch.bfloat16, 72, 40, 60)])
+def test_chained_projections(emu_ops, dtype, D, F, T):
+    util.check_chained_projections(emu_ops, dtype=dtype, T=T, D=D, F=F)
 
 
-@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 128, 128), (torch.bfloat16, 128, 128), (torch.bfloat16, 72, 40)])
-def test_clipped_input_for_the_weight_gradient(emu_ops, dtype, D, F):
-    util.check_clipped_input_output(emu_ops, dtype=dtype, T=60, D=D, F=F)
+@pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 128, 128, 60), (torch.bfloat16, 128, 128, 60),
+                                         (torch.bfloat16, 72, 40, 60)])
+def test_clipped_input_for_the_weight_gradient(emu_ops, dtype, D, F, T):
+    util.check_clipped_input_output(emu_ops, dtype=dtype, T=T, D=D, F=F)

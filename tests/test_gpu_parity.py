@@ -148,16 +148,18 @@ def test_row_chunked_weight_gradient(ops, dtype):
     util.check_row_chunked_wgrad(ops, device="cuda", dtype=dtype, T=4000)
 
 
-@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 256, 128), (torch.bfloat16, 256, 128), (torch.bfloat16, 72, 40),
-                                       (torch.float32, 100, 36)])
-def test_chained_projections(ops, dtype, D, F):
-    util.check_chained_projections(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)
+@pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 256, 128, 700), (torch.bfloat16, 256, 128, 700),
+                                         (torch.bfloat16, 72, 40, 700), (torch.float32, 100, 36, 700),
+                                         (torch.bfloat16, 256, 256, 1000), (torch.bfloat16, 512, 256, 1000)])
+def test_chained_projections(ops, dtype, D, F, T):
+    util.check_chained_projections(ops, device="cuda", dtype=dtype, T=T, D=D, F=F)
 
 
-@pytest.mark.parametrize("dtype,D,F", [(torch.float32, 256, 128), (torch.bfloat16, 256, 128), (torch.bfloat16, 256, 192),
-                                       (torch.bfloat16, 72, 40)])
-def test_clipped_input_for_the_weight_gradient(ops, dtype, D, F):
-    util.check_clipped_input_output(ops, device="cuda", dtype=dtype, T=700, D=D, F=F)
+@pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 256, 128, 700), (torch.bfloat16, 256, 128, 700),
+                                         (torch.bfloat16, 256, 192, 700), (torch.bfloat16, 72, 40, 700),
+                                         (torch.bfloat16, 256, 256, 1000), (torch.bfloat16, 256, 512, 1000)])
+def test_clipped_input_for_the_weight_gradient(ops, dtype, D, F, T):
+    util.check_clipped_input_output(ops, device="cuda", dtype=dtype, T=T, D=D, F=F)
 
 
 @pytest.mark.parametrize("name,T,D,E,F,k,routing", [("config3", 16384, 1024, 64, 256, 8, "uniform"),
