@@ -448,19 +448,18 @@ int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate
   if (!z || !dy || !grad_gate) return AMOE_ENULL;
   const size_t es = esize(dtype);
   if (!aligned(z, es) || !aligned(dy, es) || !aligned(grad_gate, es)) return AMOE_EALIGN;
-  const long long rows = (long long)T * k;
-  const long long blocks = (rows + 3) / 4;
+  const long long blocks = ((long long)T + 3) / 4;            // one wave per token
   if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   const int vec = aligned(z, 16) && aligned(dy, 16) && (D % (dtype == AMOE_F32 ? 4 : 8) == 0);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == AMOE_F32) {
     auto kf = &gate_grad_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
-                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), rows, (int)k, (int)D, vec);
+                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), (long long)T, (int)k, (int)D, vec);
   } else {
     auto kf = &gate_grad_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
-                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), rows, (int)k, (int)D, vec);
+                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), (long long)T, (int)k, (int)D, vec);
   }
   return launch_rc();
 }

@@ -757,23 +757,35 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         __syncthreads();
         constexpr int OCPR = kTileCols / CH;            // 16-byte chunks per row
         constexpr int ORPP = kThreads / OCPR;
+        // (all LDS reads of a thread first, then its stores: one wait instead of one per row)
+        constexpr int NROW = OUT_ROWS / ORPP;
+        {
+          Raw seg[NROW];
+          int orow[NROW];
 #pragma unroll
-        for (int i = 0; i < OUT_ROWS / ORPP; i++) {
-          const int rl = tid / OCPR + ORPP * i;
-          const int orow = sOrow[h * OUT_ROWS + rl];
-          if (orow >= 0)
-            *reinterpret_cast<Raw*>(DST + (int64_t)orow * ldd + c0 + (tid % OCPR) * CH) =
-                *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+          for (int i = 0; i < NROW; i++) {
+            const int rl = tid / OCPR + ORPP * i;
+            orow[i] = sOrow[h * OUT_ROWS + rl];
+            seg[i] = *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+          }
+#pragma unroll
+          for (int i = 0; i < NROW; i++)
+            if (orow[i] >= 0) *reinterpret_cast<Raw*>(DST + (int64_t)orow[i] * ldd + c0 + (tid % OCPR) * CH) = seg[i];
         }
         if (xf_stage && p.xc_out != nullptr) {     // the parked input tile, clipped and scaled in place
           const T* __restrict__ sXF = sStage + (sOut == sStage ? STAGE : 0);
+          Raw seg[NROW];
+          int xrow[NROW];
 #pragma unroll
-          for (int i = 0; i < OUT_ROWS / ORPP; i++) {
+          for (int i = 0; i < NROW; i++) {
             const int rl = tid / OCPR + ORPP * i;
-            if (row0 + rl < row_end)
-              *reinterpret_cast<Raw*>(static_cast<T*>(p.xc_out) + (int64_t)sXrow[rl] * p.ldxc + c0 + (tid % OCPR) * CH) =
-                  *reinterpret_cast<const Raw*>(&sXF[rl * LDO + (tid % OCPR) * CH]);
+            xrow[i] = row0 + rl < row_end ? sXrow[rl] : -1;
+            seg[i] = *reinterpret_cast<const Raw*>(&sXF[rl * LDO + (tid % OCPR) * CH]);
           }
+#pragma unroll
+          for (int i = 0; i < NROW; i++)
+            if (xrow[i] >= 0)
+              *reinterpret_cast<Raw*>(static_cast<T*>(p.xc_out) + (int64_t)xrow[i] * p.ldxc + c0 + (tid % OCPR) * CH) = seg[i];
         }
         __syncthreads();
       }

@@ -37,30 +37,46 @@ __global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restri
   }
 }
 
-// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>, one wave per row, 16-byte chunks per lane.
+// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>.  One wave per token: a lane's chunk of dy[t] is loaded once and
+// meets the same chunk of up to 8 head rows, whose loads are all in flight together.  Per row the sum runs
+// over the lane's chunks in ascending order, then over the lanes by a butterfly: independent of k.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict__ z, const T* __restrict__ dy,
-                                                              T* __restrict__ out, long long rows, int k, int D,
+                                                              T* __restrict__ out, long long tokens, int k, int D,
                                                               int vec) {
-  constexpr int CH = Elem<T>::kChunk;
+  constexpr int CH = Elem<T>::kChunk, JB = 8;
   const int lane = threadIdx.x & 63;
-  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  float s = 0.f;
-  if (row < rows) {
-    const T* zr = z + row * (long long)D;
-    const T* dr = dy + (row / k) * (long long)D;
+  const long long t = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= tokens) return;
+  const T* dr = dy + t * (long long)D;
+  for (int j0 = 0; j0 < k; j0 += JB) {
+    float s[JB];
+#pragma unroll
+    for (int jj = 0; jj < JB; jj++) s[jj] = 0.f;
     for (int d = lane * CH; d < D; d += 64 * CH) {
       const int nv = D - d < CH ? D - d : CH;
-      float a[CH], b[CH];
-      raw_unpack<T>(raw_load<T>(zr + d, nv, vec != 0), a);
+      Raw ra[JB];
+#pragma unroll
+      for (int jj = 0; jj < JB; jj++)
+        ra[jj] = j0 + jj < k ? raw_load<T>(z + (t * k + j0 + jj) * (long long)D + d, nv, vec != 0) : raw_zero();
+      float b[CH];
       raw_unpack<T>(raw_load<T>(dr + d, nv, vec != 0), b);
 #pragma unroll
-      for (int q = 0; q < CH; q++) s += a[q] * b[q];
+      for (int jj = 0; jj < JB; jj++) {
+        float a[CH];
+        raw_unpack<T>(ra[jj], a);
+#pragma unroll
+        for (int q = 0; q < CH; q++) s[jj] += a[q] * b[q];
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < JB; jj++) {
+      float v = s[jj];
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) v += wave_shfl_xor(v, d);
+      if (lane == 0 && j0 + jj < k) out[t * k + j0 + jj] = Elem<T>::cvt(v);
     }
   }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
-  if (row < rows && lane == 0) out[row] = Elem<T>::cvt(s);
 }
 
 template <typename T>
