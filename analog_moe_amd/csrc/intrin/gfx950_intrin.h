@@ -85,11 +85,5 @@ __device__ __forceinline__ float fast_cos_rev(float x) { return __builtin_amdgcn
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 __device__ __forceinline__ uint32_t umulhi32(uint32_t a, uint32_t b) { return __umulhi(a, b); }
-// The instruction scheduler moves nothing across this point (keeps unrolled loops from hoisting all their
-// loads to the top and running out of registers).
-__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
-// The same value, but the optimiser cannot see that: whatever is computed from it is computed where it is
-// used instead of being hoisted out of the enclosing loops into registers that then stay occupied.
-__device__ __forceinline__ int opaque_copy(int v) { asm volatile("" : "+v"(v)); return v; }
 
 }  // namespace amoe

@@ -131,8 +131,6 @@ inline float fast_sin_rev(float x) { return sinf(6.283185307179586f * x); }
 inline float fast_cos_rev(float x) { return cosf(6.283185307179586f * x); }
 inline int wave_uniform(int v) { return v; }
 inline float fast_log2(float x) { return log2f(x); }
-inline void sched_fence() {}
-inline int opaque_copy(int v) { return v; }
 inline float fast_sqrt(float x) { return sqrtf(x); }
 inline uint32_t umulhi32(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
 
