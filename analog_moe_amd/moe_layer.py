@@ -114,7 +114,7 @@ class SigmaMoELayer(nn.Module):
         """Gate values and expert ids [..., k] of the top-k experts, and the regularisation loss."""
         logits = self.expert_sel(x)
         reg_loss = x.new_zeros(())
-        if self.training:
+        if self.training and logits.numel() > 0:
             logp = F.log_softmax(logits.float(), dim=-1).flatten(end_dim=-2)
             mean_logp = torch.logsumexp(logp, dim=0) - math.log(logp.shape[0])
             reg_loss = (mean_logp.exp() * mean_logp).sum()          # minus entropy of the mean usage

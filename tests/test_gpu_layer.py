@@ -440,3 +440,33 @@ def test_clip_types_run(kind):
     bound = 2.0 * before.std(dims, keepdim=True)
     assert torch.equal(layer.keys.detach(), torch.minimum(torch.maximum(before, -bound), bound))
     assert not torch.equal(layer.keys, before)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("tokens", [0, 1])
+def test_empty_and_single_token_batches(fused, tokens):
+    """No tokens at all: empty output, zero weight gradients, nothing launched on missing rows; one token: k
+    experts own one row each and every other expert's gradient tile is written as zeros."""
+    from analog_moe_amd import config as cfgmod
+    mods = {} if fused else {"bias": True}
+    layer = _layer(cfgmod, mods, decay=0.01, out_bound=12.0, out_res=254)
+    assert layer._fusable() == fused
+    layer.train()
+    x = torch.randn(tokens, 3, 128, device="cuda", requires_grad=True)
+    y, reg = layer(x)
+    assert y.shape == x.shape
+    (y.sum() + reg).backward()
+    torch.cuda.synchronize()
+    assert x.grad.shape == x.shape and torch.isfinite(layer.keys.grad).all() and torch.isfinite(layer.values.grad).all()
+    if tokens == 0:
+        assert layer.keys.grad.abs().sum() == 0 and layer.values.grad.abs().sum() == 0
+    else:
+        _, sel_idx, _ = layer.select(x.detach())
+        unused = [e for e in range(layer.n_experts) if e not in set(sel_idx.reshape(-1).tolist())]
+        for e in unused:
+            assert layer.keys.grad[e].abs().sum() == 0 and layer.values.grad[e].abs().sum() == 0
+        want = _oracle_for(layer, x, *[t.detach() for t in layer.select(x.detach())[:2]], torch.ones_like(y),
+                           inp_res=1 / 127, decay=0.01, input_min_percentage=0.5, out_bound=12.0, out_res=254.0,
+                           wmax_up=util.np32(layer.keys.abs().amax((1, 2)).reshape(-1, 1)),
+                           wmax_down=util.np32(layer.values.abs().amax((1, 2)).reshape(-1, 1)))
+        assert util.rel_err(util.np32(y).reshape(-1, 128), want.y) < 2e-3      # (an ADC step where codes tie)
