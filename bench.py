@@ -31,6 +31,11 @@ CONFIGS = {
                name="config3: d_model=1024 (2x512 tiles) E=64 F=256 k=8 16384 tokens bf16 uniform routing"),
     "c4": dict(T=32768, D=2048, E=128, F=512, k=4, dtype="bf16", routing="zipf", mis=-1, noise=0.04,
                name="config4: d_model=2048 E=128 F=512 k=4 32768 tokens bf16 Zipf(1.2) routing"),
+    # the layer inside its caller: a 16-layer decoder training step (attention and norms are stock PyTorch)
+    "c5": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="bf16", routing="router", mis=-1, noise=0.04,
+               layers=16, heads=16, context=1024, batch=16, vocab=8000,
+               name="config5: 16-layer SigmaMoE decoder training step, d_model=1024, 16 heads, 64 experts x 256, "
+                    "k=8, context 1024, batch 16, vocab 8000, bf16"),
 }
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
@@ -82,6 +87,90 @@ def cpu_baseline(cfg, pr, budget_tokens):
                       f"{dt * 1e3:.1f} ms each"}
 
 
+def bench_decoder(args, cfg):
+    """Configuration 5: forward, loss, backward and optimizer step of a 16-layer SigmaMoE decoder whose
+    feed-forward blocks are the analog layer.  Reports whole-step tokens/s and, from a second timing with the
+    feed-forward blocks switched off, the share and the TFLOP/s of the MoE part."""
+    import torch
+    from torch import nn
+    from analog_moe_amd import config as cfgmod, ops
+    from analog_moe_amd.decoder import SigmaMoEDecoder
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayer
+
+    ops.get_lib()
+    dev = torch.device("cuda:0")
+    D, E, F, k = (cfg[n] for n in "DEFk")
+    B, S, V, L = cfg["batch"], cfg["context"], cfg["vocab"], cfg["layers"]
+
+    def rpu():
+        r = cfgmod.TorchInferenceRPUConfig()
+        r.forward.inp_res = r.forward.out_res = 2 ** 8 - 2
+        r.forward.out_bound = 12.0
+        r.forward.out_noise = cfg["noise"]
+        r.pre_post.input_range.enable = True
+        r.pre_post.input_range.learn_input_range = True
+        r.pre_post.input_range.init_value = 3.0
+        r.pre_post.input_range.decay = 0.01
+        return r
+
+    class NoFFN(nn.Module):
+        def forward(self, x):
+            return torch.zeros_like(x), x.new_zeros(())
+
+    def build(with_moe):
+        torch.manual_seed(0)
+        make = (lambda i: AnalogSigmaMoELayer(rpu(), d_model=D, n_experts=E, expert_size=F, k=k)) if with_moe \
+            else (lambda i: NoFFN())
+        model = SigmaMoEDecoder(V, D, L, cfg["heads"], S, make).to(dev).to(torch.bfloat16)
+        model.train()
+        for blk in model.blocks:
+            if with_moe:
+                blk.ffn.use_device_noise_counter()
+        return model
+
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, V, (B, S), generator=g).to(dev)          # uniform random token ids
+    labels = torch.roll(ids, -1, dims=1)
+
+    def timed(model):
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+
+        def step():
+            loss, _ = model(ids, labels, reg_weight=0.01)
+            loss.backward()
+            opt.step()
+            model.post_update_step()
+            opt.zero_grad(set_to_none=True)
+            return loss.detach()
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            last = step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3, float(last.detach())
+
+    ms, loss = timed(build(True))
+    ms_rest, _ = timed(build(False))
+    T = B * S
+    moe_ms = ms - ms_rest
+    moe_flops = L * 12.0 * T * k * D * F
+    out = {
+        "metric": "SigmaMoE decoder HWA training step tokens/sec on 1 GPU", "value": T / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg["name"], "optimizer": "AdamW", "launch": "eager",
+                   "analog": "learned input range 3.0, 8-bit DAC, 8-bit ADC (out_bound 12), output noise 0.04 x "
+                             "max|W| drawn in-kernel; router digital"},
+        "loss_after_last_step": loss,
+        "ms_per_step_without_ffn": ms_rest, "moe_part_ms": moe_ms, "moe_part_share": moe_ms / ms,
+        "moe_part_tflops": moe_flops / (moe_ms * 1e-3) / 1e12,
+        "moe_part_pct_of_mfma_peak": 100.0 * moe_flops / (moe_ms * 1e-3) / PEAK["bf16"],
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -104,6 +193,8 @@ def main():
     from tests import util
 
     cfg = CONFIGS[args.config]
+    if "layers" in cfg:
+        return bench_decoder(args, cfg)
     ops.get_lib()
     dev = torch.device("cuda:0")
     tdt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32

@@ -470,3 +470,42 @@ def test_empty_and_single_token_batches(fused, tokens):
                            wmax_up=util.np32(layer.keys.abs().amax((1, 2)).reshape(-1, 1)),
                            wmax_down=util.np32(layer.values.abs().amax((1, 2)).reshape(-1, 1)))
         assert util.rel_err(util.np32(y).reshape(-1, 128), want.y) < 2e-3      # (an ADC step where codes tie)
+
+
+def test_decoder_training_step():
+    """The layer inside its caller (a small SigmaMoE decoder): the feed-forward of a block sees exactly what the
+    stand-alone layer computes, gradients reach every parameter of every block, and a few optimizer steps on
+    one batch bring the loss down."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.decoder import SigmaMoEDecoder
+    torch.manual_seed(0)
+    layers = []
+
+    def make(i):
+        layers.append(_layer(cfgmod, {}, decay=0.01, out_bound=12.0, out_res=254))
+        return layers[-1]
+    model = SigmaMoEDecoder(vocab_size=97, d_model=128, n_layers=2, n_heads=4, context=32, make_ffn=make).cuda()
+    model.train()
+    ids = torch.randint(0, 97, (4, 32), device="cuda")
+    labels = torch.roll(ids, -1, dims=1)
+    # the block's feed-forward output equals the stand-alone layer on the same input
+    seen = {}
+    h = model.blocks[1].ffn.register_forward_hook(lambda m, a, out: seen.update(x=a[0].detach(), y=out[0].detach()))
+    logits, reg = model(ids)
+    h.remove()
+    assert logits.shape == (4, 32, 97) and torch.isfinite(logits).all()
+    alone, _ = layers[1](seen["x"])
+    assert torch.equal(alone, seen["y"])
+    opt = torch.optim.AdamW(model.parameters(), lr=3e-3)
+    losses = []
+    for _ in range(8):
+        loss, _ = model(ids, labels, reg_weight=0.01)
+        loss.backward()
+        if not losses:
+            missing = [n for n, p in model.named_parameters() if p.requires_grad and p.grad is None]
+            assert missing == []
+        opt.step()
+        model.post_update_step()
+        opt.zero_grad(set_to_none=True)
+        losses.append(float(loss.detach()))
+    assert losses[-1] < 0.8 * losses[0]
