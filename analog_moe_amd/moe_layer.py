@@ -12,7 +12,8 @@ test_moe_layer_aihwkit_lightning.py:82-107).
 Differences from the reference, all opt-in through ``rpu_config``: ``mapping.max_input_size``
 (K-tile split with one input range per tile), ``forward.out_bound`` / ``out_res`` (ADC) are
 implemented instead of asserted off (:152-160); output noise is drawn inside the kernel unless
-``noise_mode="injected"`` is chosen.  The router stays a digital ``nn.Linear``.
+``noise_mode="injected"`` is chosen.  The router is an analog linear layer on the same kernels
+(``AnalogLinear``; ``analog_router=False`` keeps a digital ``nn.Linear``).
 """
 from __future__ import annotations
 
@@ -151,6 +152,126 @@ class SigmaMoELayer(nn.Module):
         return self.forward_selected(x, sel_val, sel_idx), reg_loss
 
 
+class AnalogLinear(nn.Module):
+    """An analog linear layer ``y = A(x) @ weight.T`` on the CVMM kernels: one analog tile per K-tile, which the
+    kernels see as a one-expert selection (every row belongs to expert 0, in order).
+
+    The reference turns the router ``expert_sel`` into an analog layer with aihwkit-lightning's
+    ``convert_to_analog`` (moe_layer_aihwkit_lightning.py:195-200), so the expert selection itself sees the
+    input range, the DAC, the output noise and the ADC.  That package is third-party; this class applies the
+    same stages with the definitions of this build (they are the expert projections' own): parameters
+    ``weight [out, in]`` as in ``nn.Linear`` (no bias), ``input_range [n_tiles]``, ``input_range_update_idx``.
+    """
+
+    def __init__(self, in_features: int, out_features: int, rpu_config, noise_mode: str = "kernel"):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.rpu_config = rpu_config
+        self.noise_mode = noise_mode
+        self.weight = nn.Parameter(torch.empty(out_features, in_features))
+        self.register_parameter("bias", None)
+        self.bounds = tile_bounds(in_features, getattr(rpu_config.mapping, "max_input_size", -1))
+        self.n_tiles = 1 if self.bounds is None else len(self.bounds) - 1
+        self.input_range = None
+        irp = rpu_config.pre_post.input_range
+        if irp.enable:
+            self.input_range_update_idx = nn.Parameter(torch.tensor(0.0), requires_grad=False)
+            ir = torch.full((self.n_tiles,), float(irp.init_value))
+            if irp.learn_input_range:
+                self.input_range = nn.Parameter(ir)
+            else:
+                del self.input_range
+                self.register_buffer("input_range", ir)
+        self._init_done = False
+        self._noise_calls = 0
+        self._noise_seed_base = 0
+        self.noise_counter: Optional[Tensor] = None
+        self._rows = {}                           # one-expert selection per row count
+
+    def _selection(self, T: int, device) -> CVMMSel:
+        def make():
+            i32 = dict(dtype=torch.int32, device=device)
+            zeros = torch.zeros(T, **i32)
+            return CVMMSel(zeros, zeros, torch.arange(T, **i32), None, None, torch.arange(2, **i32) * T)
+        if torch.compiler.is_compiling():
+            return make()
+        key = (T, str(device))
+        if key not in self._rows:
+            self._rows[key] = make()
+        return self._rows[key]
+
+    def _init_pending(self) -> bool:
+        n = self.rpu_config.pre_post.input_range.init_from_data
+        if n <= 0 or self._init_done:
+            return False
+        if not bool(self.input_range_update_idx < n):
+            self._init_done = True
+            return False
+        return True
+
+    def _seed(self) -> int:
+        salt = 0x5851F42D4C957F2D                  # a seed stream of its own, apart from the expert projections'
+        if self.noise_counter is not None:
+            return (self._noise_seed_base ^ salt) & (2 ** 63 - 1)
+        if torch.compiler.is_compiling():
+            raise MoEConifgError("a compiled noisy forward would freeze the host-side noise seed: call "
+                                 "use_device_noise_counter() on the layer before torch.compile")
+        self._noise_calls += 1
+        return ((torch.initial_seed() * 0x9E3779B97F4A7C15 + self._noise_calls * 0xD1B54A32D192ED03) ^ salt) \
+            & (2 ** 63 - 1)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if not (x.is_cuda or x.is_meta):
+            raise MoEConifgError("Analog MoE executed on CPU. This package runs on the GPU only.")
+        fwd = self.rpu_config.forward
+        irp = self.rpu_config.pre_post.input_range
+        x2 = x.reshape(-1, self.in_features)
+        sel = self._selection(x2.shape[0], x.device)
+        perfect = bool(getattr(fwd, "is_perfect", False))
+        bir = None
+        if self.input_range is not None:
+            if self.training and self._init_pending():
+                std = cvmm_std(x2, sel.sel_index, sel.sel, 1).float()
+                if bool(std[0] > 0):
+                    idx = self.input_range_update_idx
+                    self.input_range.data = ((self.input_range.data * idx + irp.init_std_alpha * std[0]) / (idx + 1)
+                                             ).abs().to(self.input_range.dtype)
+                    self.input_range_update_idx.data += 1
+            bir = self.input_range.reshape(1, self.n_tiles).expand(x2.shape[0], self.n_tiles)
+        w = self.weight.t().unsqueeze(0)                               # [1, in, out]: a transposed view
+        modified = w
+        if (self.training or self.rpu_config.modifier.enable_during_test) and \
+                enum_name(self.rpu_config.modifier.type) not in ("NONE", "COPY"):
+            modified = AnalogSigmaMoELayer.modify_weight(w.clone(), self.rpu_config.modifier)
+        ext = AnalogExt(offsets=sel.offsets, bounds=self.bounds,
+                        out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
+                        out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
+        per_channel = bool(getattr(fwd, "out_noise_per_channel", False))
+        noisy = self.training and fwd.out_noise > 0 and not perfect
+        if ext.out_bound > 0 or noisy:
+            ext.wmax = torch.ops.amoe.weight_abs_max(w.detach().contiguous(), per_channel)
+        out_noise = None
+        if noisy and self.noise_mode == "kernel":
+            ext.noise_std, ext.noise_seed, ext.noise_seed_dev = float(fwd.out_noise), self._seed(), self.noise_counter
+        elif noisy:
+            out_noise = torch.randn(self.n_tiles, x2.shape[0], self.out_features, device=x.device) \
+                * fwd.out_noise * ext.wmax[0]
+        y = CVMM.apply(x2, sel.sel_index, sel.sel, modified, -1.0 if perfect else kernel_inp_res(fwd.inp_res), bir,
+                       None, None, out_noise, irp, fwd, ext)
+        return y.view(*x.shape[:-1], self.out_features)
+
+    @torch.no_grad()
+    def clip_weights(self) -> None:
+        kind = enum_name(self.rpu_config.clip.type)
+        if kind in ("LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL"):
+            dims = None if kind == "LAYER_GAUSSIAN" else 1
+            bound = self.rpu_config.clip.sigma * (self.weight.std() if dims is None else self.weight.std(1, keepdim=True))
+            self.weight.data = torch.minimum(torch.maximum(self.weight.data, -bound), bound)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, tiles={self.n_tiles}"
+
+
 def load_state_dict_pre_hook(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
     """Accept checkpoints written by the traceable layout (per-expert ``keys.{i}.input_range``
     entries, moe_layer_aihwkit_lightning.py:66-105) by folding them into ``input_range [2, E]``."""
@@ -186,12 +307,16 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     the reference does (:472-492) and hands them to the kernel."""
 
     def __init__(self, rpu_config: Optional[TorchInferenceRPUConfig] = None, *args, noise_mode: str = "kernel",
-                 **kwargs):
+                 analog_router: bool = True, **kwargs):
         super().__init__(*args, **kwargs)
         self.rpu_config = TorchInferenceRPUConfig() if rpu_config is None else rpu_config
         if noise_mode not in ("kernel", "injected"):
             raise MoEConifgError("noise_mode must be 'kernel' or 'injected'")
         self.noise_mode = noise_mode
+        if analog_router:                  # moe_layer_aihwkit_lightning.py:195-200: the router is analog too
+            digital = self.expert_sel
+            self.expert_sel = AnalogLinear(self.k_dim, self.n_experts, self.rpu_config, noise_mode)
+            self.expert_sel.weight.data = digital.weight.data.clone()
         self._noise_calls = 0
         self._noise_seed_base = 0
         self._init_done = False            # host-side latch of "input_range_update_idx reached init_from_data"
@@ -235,7 +360,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
                               sinkhorn_n_iters=module.sinkhorn_n_iters, expert_dropout=module.expert_dropout)
         layer.keys.data = module.keys.data.detach().clone()
         layer.values.data = module.values.data.detach().clone()
-        layer.expert_sel.load_state_dict(module.expert_sel.state_dict())
+        layer.expert_sel.weight.data = module.expert_sel.weight.data.detach().clone()
         if module.bias is not None:
             layer.bias.data = module.bias.data.detach().clone()
             layer.o_bias.data = module.o_bias.data.detach().clone()
@@ -295,6 +420,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     def post_update_step(self) -> None:
         if hasattr(self.rpu_config, "clip") and enum_name(self.rpu_config.clip.type) != "NONE":
             self.clip_weights()
+            if isinstance(self.expert_sel, AnalogLinear):
+                self.expert_sel.clip_weights()
 
     @torch.no_grad()
     def clip_weights(self) -> None:
@@ -347,6 +474,9 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             self.noise_counter = torch.zeros(1, dtype=torch.int64, device=self.keys.device)
         # the host part of the seed is read here, once: a traced or captured forward cannot ask for it
         self._noise_seed_base = (torch.initial_seed() * 0x9E3779B97F4A7C15) & (2 ** 63 - 1)
+        if isinstance(self.expert_sel, AnalogLinear):       # the router draws from the same counter
+            self.expert_sel.noise_counter = self.noise_counter
+            self.expert_sel._noise_seed_base = self._noise_seed_base
         return self.noise_counter
 
     def _noise_seed(self) -> int:
@@ -483,6 +613,9 @@ class AnalogSigmaMoELayerAIHWKIT(AnalogSigmaMoELayer):
                                  "(an aihwkit TorchInferenceRPUConfig or AIHWKITTorchInferenceRPUConfig)")
         assert getattr(fwd, "inp_bound", 1.0) in [-1, 1.0], "inp_bound must be 1.0 or off (=-1)"
         assert enum_name(getattr(fwd, "bound_management", "NONE")) == "NONE", "bound_management must be NONE"
+        # this flavour keeps the router it is given (moe_layer_aihwkit.py:88-94, 135-142): converting it is left
+        # to the caller's conversion of the whole model
+        kwargs.setdefault("analog_router", False)
         super().__init__(rpu_config, *args, **kwargs)
 
     # -- flavour hooks ---------------------------------------------------------------------------------------

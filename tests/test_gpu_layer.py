@@ -509,3 +509,45 @@ def test_decoder_training_step():
         opt.zero_grad(set_to_none=True)
         losses.append(float(loss.detach()))
     assert losses[-1] < 0.8 * losses[0]
+
+
+def test_analog_router_is_an_analog_linear_layer():
+    """The router goes through the same analog stages as an expert projection (the reference converts it with
+    convert_to_analog, moe_layer_aihwkit_lightning.py:195-200): as a one-expert CVMM its logits are the oracle's
+    clip / DAC / matmul / ADC of x against weight.T, and weight, input range and input all get gradients that
+    follow the closed forms (straight-through rounding, strict clip mask)."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.moe_layer import AnalogLinear
+    layer = _layer(cfgmod, {}, decay=0.0, out_bound=12.0, out_res=254)
+    router = layer.expert_sel
+    assert isinstance(router, AnalogLinear) and router.input_range.shape == (1,)
+    with torch.no_grad():
+        router.input_range.fill_(1.5)
+    x = torch.randn(6, 10, 128, device="cuda", requires_grad=True)
+    layer.eval()
+    logits = router(x)
+    assert logits.shape == (6, 10, 4)
+    x2 = util.np32(x.reshape(-1, 128))
+    w = util.np32(router.weight.t().unsqueeze(0))                      # [1, 128, 4]
+    rows = np.arange(60, dtype=np.int32)
+    zeros = np.zeros(60, dtype=np.int32)
+    wmax = np.abs(w).max().reshape(1, 1)
+    want = O.cvmm_fwd(x2, rows, zeros, w, inp_res=1 / 127, ir=np.full((60, 1), 1.5, np.float32), wmax=wmax,
+                      out_bound=12.0, out_res=254.0)
+    step = 2 * 12.0 * float(wmax[0, 0]) / 254 * 1.5
+    assert np.abs(util.np32(logits).reshape(60, 4) - want).max() <= step * 1.001     # at most one ADC step where codes tie
+    assert np.mean(np.abs(util.np32(logits).reshape(60, 4) - want) > 1e-5) < 0.02
+    # gradients: d logits / d weight is the clipped input, the clip mask gates d / dx
+    g = torch.randn_like(logits)
+    logits.backward(g)
+    clipped = np.clip(x2, -1.5, 1.5)
+    assert util.rel_err(util.np32(router.weight.grad), (clipped.T @ util.np32(g).reshape(60, 4)).T) < 1e-5
+    gx = (util.np32(g).reshape(60, 4) @ util.np32(router.weight)) * (np.abs(x2) < 1.5)
+    assert util.rel_err(util.np32(x.grad).reshape(60, 128), gx) < 1e-5
+    assert router.input_range.grad is not None and router.input_range.grad.abs() > 0
+    # a digital router is still available, and the whole layer trains through the analog one
+    assert isinstance(_layer(cfgmod, {"analog_router": False}).expert_sel, torch.nn.Linear)
+    layer.train()
+    y, reg = layer(x.detach())
+    (y.sum() + reg).backward()
+    assert torch.isfinite(router.weight.grad).all()

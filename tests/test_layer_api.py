@@ -31,7 +31,11 @@ def test_constructor_and_state_dict_keys():
     assert layer.keys.shape == (4, 32, 16) and layer.values.shape == (4, 16, 32)
     assert layer.input_range.shape == (2, 4) and isinstance(layer.input_range, torch.nn.Parameter)
     sd = layer.state_dict()
-    assert set(sd) == {"keys", "values", "expert_sel.weight", "input_range", "input_range_update_idx"}
+    assert set(sd) == {"keys", "values", "input_range", "input_range_update_idx", "expert_sel.weight",
+                       "expert_sel.input_range", "expert_sel.input_range_update_idx"}     # the router is analog too
+    digital_router = AnalogSigmaMoELayer(_rpu(), d_model=32, n_experts=4, expert_size=16, k=2, analog_router=False)
+    assert set(digital_router.state_dict()) == {"keys", "values", "expert_sel.weight", "input_range",
+                                                "input_range_update_idx"}
     assert sd._metadata[""]["rpu_config"] is layer.rpu_config
     fixed = AnalogSigmaMoELayer(_rpu(learn=False), d_model=32, n_experts=4, expert_size=16, k=2)
     assert not isinstance(fixed.input_range, torch.nn.Parameter) and "input_range" in fixed.state_dict()
