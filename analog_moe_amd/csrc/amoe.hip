@@ -307,7 +307,8 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   }
   const long long grid = 8LL * ((pairs + 7) / 8) * p.n_k_blocks * p.n_n_blocks;   // see the id mapping in the kernel
   if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
-  const long long rgrid = (long long)a->E * p.n_k_blocks * p.n_n_blocks;
+  const long long rgrid = (long long)a->E * p.n_k_blocks * p.n_n_blocks * kWgradReduceSplit;
+  if (rgrid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   if (a->dtype == AMOE_F32) {
     auto k = &gemm_wgrad_kernel<float>;
     hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);

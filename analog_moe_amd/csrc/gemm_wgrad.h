@@ -354,14 +354,17 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   }
 }
 
-// Second launch of a row-chunked weight gradient: one workgroup per (expert, tile) adds the fp32
-// partial tiles of a multi-chunk expert in chunk order and writes the tile of grad_w.
+// Second launch of a row-chunked weight gradient: kWgradReduceSplit workgroups per (expert, tile), each
+// with its share of the tile's rows, add the fp32 partial tiles of a multi-chunk expert in chunk order and
+// write the tile of grad_w.
+constexpr int kWgradReduceSplit = 8;
 template <typename T>
 __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(const WgradParams p) {
   __shared__ int sSum[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tiles = p.n_k_blocks * p.n_n_blocks;
-  const int e = blockIdx.x / tiles, tile_id = blockIdx.x % tiles;
+  const int part = blockIdx.x % kWgradReduceSplit, et = blockIdx.x / kWgradReduceSplit;
+  const int e = et / tiles, tile_id = et % tiles;
   const int R = p.rows_per_chunk;
   const int n_chunks = wgrad_chunks(p.offsets[e + 1] - p.offsets[e], R);
   if (n_chunks <= 1) return;
@@ -380,12 +383,21 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(const WgradParam
   const int n0 = nb * kTileCols;
   const float* __restrict__ first = p.partial + ((int64_t)slot0 * tiles + tile_id) * kWgradTileElems;
   T* __restrict__ GW = static_cast<T*>(p.grad_w) + (int64_t)e * p.K * p.N;
-  for (int it = 0; it < kWgradTileElems / (4 * kThreads); it++) {
-    const int idx = (it * kThreads + tid) * 4;
+  constexpr int kIters = kWgradTileElems / (4 * kThreads * kWgradReduceSplit);
+  const int64_t cstride = (int64_t)tiles * kWgradTileElems;
+  for (int it = 0; it < kIters; it++) {
+    const int idx = ((part * kIters + it) * kThreads + tid) * 4;
     const int row = idx / kTileCols, col = idx % kTileCols;
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < n_chunks; c++)
-      sum += *reinterpret_cast<const f32x4*>(&first[(int64_t)c * tiles * kWgradTileElems + idx]);
+    int c = 0;
+    for (; c + 4 <= n_chunks; c += 4) {      // four loads in flight, added in chunk order
+      f32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const f32x4*>(&first[(c + u) * cstride + idx]);
+#pragma unroll
+      for (int u = 0; u < 4; u++) sum += v[u];
+    }
+    for (; c < n_chunks; c++) sum += *reinterpret_cast<const f32x4*>(&first[c * cstride + idx]);
     const int kk = kcol.c0 + row, n = n0 + col;
     int nv = kk < kcol.c1 ? p.N - n : 0;
     nv = nv < 0 ? 0 : (nv > 4 ? 4 : nv);
