@@ -162,7 +162,7 @@ def bench_decoder(args, cfg):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": cfg["name"], "optimizer": "AdamW", "launch": "eager",
                    "analog": "learned input range 3.0, 8-bit DAC, 8-bit ADC (out_bound 12), output noise 0.04 x "
-                             "max|W| drawn in-kernel; router digital"},
+                             "max|W| drawn in-kernel; analog router"},
         "loss_after_last_step": loss,
         "ms_per_step_without_ffn": ms_rest, "moe_part_ms": moe_ms, "moe_part_share": moe_ms / ms,
         "moe_part_tflops": moe_flops / (moe_ms * 1e-3) / 1e12,
