@@ -402,7 +402,10 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         kind = enum_name(modifier.type)
         if kind == "NONE":
             return inp_weight
-        if kind.endswith("PER_CHANNEL"):
+        # per-channel max |W| for the two discretising per-channel types only: the reference's list
+        # (moe_layer_aihwkit_lightning.py:333-337) names DISCRETIZE_ADD_NORMAL_PER_CHANNEL twice and leaves
+        # ADD_NORMAL_PER_CHANNEL out, so that type scales its noise by the per-expert maximum -- kept as it is
+        if kind in ("DISCRETIZE_PER_CHANNEL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL"):
             wmax = inp_weight.abs().amax(1, keepdim=True)
         else:
             wmax = inp_weight.reshape(inp_weight.size(0), -1).abs().amax(-1).view(-1, 1, 1)

@@ -92,6 +92,15 @@ def test_inp_res_mapping_and_weight_modifier():
     assert torch.allclose(q / step, torch.round(q / step), atol=1e-4)
     m2 = cfg.WeightModifierParameter(type=cfg.WeightModifierType.ADD_NORMAL, std_dev=0.1)
     assert not torch.equal(AnalogSigmaMoELayer.modify_weight(w.clone(), m2), w)
+    # ADD_NORMAL_PER_CHANNEL scales its noise by the per-expert maximum, as the reference's type list makes it
+    # (moe_layer_aihwkit_lightning.py:333-337): a quiet channel gets the same noise as a loud one
+    torch.manual_seed(0)
+    wq = torch.randn(2, 256, 6)
+    wq[:, :, 0] *= 20
+    m3 = cfg.WeightModifierParameter(type=cfg.WeightModifierType.ADD_NORMAL_PER_CHANNEL, std_dev=0.1)
+    d = AnalogSigmaMoELayer.modify_weight(wq.clone(), m3) - wq
+    assert d[:, :, 0].std() == pytest.approx(d[:, :, 1:].std().item(), rel=0.2)
+    assert d[0].std() == pytest.approx(0.1 * wq[0].abs().max().item(), rel=0.15)
     layer = AnalogSigmaMoELayer(_rpu(), d_model=8, n_experts=3, expert_size=5, k=1)
     layer.rpu_config.clip.type = cfg.WeightClipType.LAYER_GAUSSIAN
     layer.rpu_config.clip.sigma = 1.0
