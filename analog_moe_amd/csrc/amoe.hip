@@ -4,6 +4,7 @@
 #include "gemm_rows.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
+#include "weight_kernels.h"
 #include "prepare_sel.h"
 
 using namespace amoe;
@@ -487,6 +488,23 @@ int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, in
   return launch_rc();
 }
 
+// Work split of the per-channel reductions over w [E, K, N]: lanes per row (a power of two covering the row's
+// 16-byte chunks, at most 64) and K slices (at least eight loads per lane, about four workgroups per CU overall).
+struct ColSplit { int width, slices, col_blocks; };
+static ColSplit col_split(int dtype, int E, int K, int N) {
+  const int CH = 16 / (int)esize(dtype);
+  const int chunks = (N + CH - 1) / CH;
+  ColSplit c;
+  c.width = 64;
+  while (c.width / 2 >= chunks) c.width /= 2;
+  const int rows_per_block = 4 * (64 / c.width);
+  const int most = (K + 8 * rows_per_block - 1) / (8 * rows_per_block);
+  const int want = (1024 + E - 1) / E;
+  c.slices = most < 1 ? 1 : (most > want ? want : most);
+  c.col_blocks = (chunks + 63) / 64;
+  return c;
+}
+
 int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* wmax,
                         void* stream) {
   if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
@@ -510,13 +528,21 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
       hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax, vec);
     }
   } else {
-    dim3 grid((N + kThreads - 1) / kThreads, E);
+    if ((long long)E * N > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(((long long)E * N + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                       st, reinterpret_cast<uint32_t*>(wmax), (int)(E * N));
+    if (int rc = launch_rc()) return rc;
+    const ColSplit cs = col_split(dtype, E, K, N);
+    const int width = cs.width;
+    const int vec = aligned(w, 16) && (N % (16 / (int)esize(dtype)) == 0);
+    dim3 grid(cs.col_blocks, cs.slices, E);
     if (dtype == AMOE_F32) {
       auto kf = &weight_col_abs_max_kernel<float>;
-      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, wmax);
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, width, wmax, vec);
     } else {
       auto kf = &weight_col_abs_max_kernel<uint16_t>;
-      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, wmax);
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, width, wmax,
+                         vec);
     }
   }
   return launch_rc();
@@ -547,6 +573,119 @@ int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K, const 
     auto kf = &expert_std_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(x), (long long)ldx, (int)K,
                        in_index, offsets, out);
+  }
+  return launch_rc();
+}
+
+int amoe_modify_weight(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, const float* wmax,
+                       int32_t wmax_cols, float n_states, float std_dev, const float* noise, int32_t round_noise,
+                       uint64_t noise_seed, const uint64_t* noise_seed_dev, void* out, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (E < 1 || K < 1 || N < 1 || (wmax_cols != 1 && wmax_cols != N)) return AMOE_EINVAL;
+  if (!w || !out || !wmax) return AMOE_ENULL;
+  if (!aligned(w, esize(dtype)) || !aligned(out, esize(dtype)) || !aligned(wmax, 4) || !aligned(noise, 4) ||
+      !aligned(noise_seed_dev, 8))
+    return AMOE_EALIGN;
+  const int CH = 16 / esize(dtype);
+  const long long rows = (long long)E * K;
+  const long long blocks = (rows * ((N + CH - 1) / CH) + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL || rows > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  ModifyParams p{};
+  p.w = w; p.out = out; p.wmax = wmax; p.noise = noise; p.rows = rows; p.K = K; p.N = N; p.wmax_cols = wmax_cols;
+  p.inv_states = n_states > 0.f ? 1.0f / n_states : 0.f; p.std_dev = std_dev; p.round_noise = round_noise; p.seed = noise_seed;
+  p.seed_dev = noise_seed_dev;
+  p.vec = aligned(w, 16) && aligned(out, 16) && (N % CH == 0);
+  p.cvec = aligned(wmax, 16) && (N % CH == 0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &modify_weight_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, p);
+  } else {
+    auto kf = &modify_weight_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, p);
+  }
+  return launch_rc();
+}
+
+static int std_slices(long long per_expert) {
+  const long long s = (per_expert + 32 * kThreads - 1) / (32 * kThreads);
+  return s < 1 ? 1 : (s > kStdMaxSlices ? kStdMaxSlices : (int)s);
+}
+
+size_t amoe_weight_std_workspace(int32_t E, int32_t K, int32_t N, int32_t cols) {
+  if (E < 1 || K < 1 || N < 1) return 0;
+  if (cols == N && N != 1) return (size_t)E * col_split(AMOE_F32, E, K, N).slices * N * 2 * sizeof(double);
+  return (size_t)E * std_slices((long long)K * N) * 2 * sizeof(double);
+}
+
+int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* std_out,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
+  if (!w || !std_out) return AMOE_ENULL;
+  if (!aligned(w, esize(dtype)) || !aligned(std_out, 4) || !aligned(workspace, 8)) return AMOE_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!workspace) return AMOE_ENULL;
+  if (workspace_bytes < amoe_weight_std_workspace(E, K, N, cols)) return AMOE_EWORKSPACE;
+  double* partial = static_cast<double*>(workspace);
+  if (cols == N && N != 1) {
+    if ((long long)E * N > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+    ColSplit cs = col_split(dtype, E, K, N);
+    const int most = col_split(AMOE_F32, E, K, N).slices;        // what the workspace was sized for
+    if (cs.slices > most) cs.slices = most;
+    const int vec = aligned(w, 16) && (N % (16 / (int)esize(dtype)) == 0);
+    dim3 grid(cs.col_blocks, cs.slices, E);
+    if (dtype == AMOE_F32) {
+      auto kf = &weight_col_moments_kernel<float>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, cs.width, partial,
+                         vec);
+    } else {
+      auto kf = &weight_col_moments_kernel<uint16_t>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, cs.width,
+                         partial, vec);
+    }
+    if (int rc = launch_rc()) return rc;
+    hipLaunchKernelGGL(weight_col_std_finalize_kernel, dim3((unsigned)(((long long)E * N + kThreads - 1) / kThreads)),
+                       dim3(kThreads), 0, st, partial, cs.slices, (int)K, (int)N, (int)E, std_out);
+    return launch_rc();
+  }
+  const long long per = (long long)K * N;
+  const int slices = std_slices(per);
+  const int vec = aligned(w, 16) && (per % 16 == 0);
+  if (dtype == AMOE_F32) {
+    auto kf = &weight_moments_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3(slices, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, partial, vec);
+  } else {
+    auto kf = &weight_moments_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3(slices, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, partial, vec);
+  }
+  if (int rc = launch_rc()) return rc;
+  hipLaunchKernelGGL(weight_std_finalize_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st, partial,
+                     slices, per, (int)E, std_out);
+  return launch_rc();
+}
+
+int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N, const float* bound, int32_t cols,
+                       void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
+  if (!w || !bound) return AMOE_ENULL;
+  if (!aligned(w, esize(dtype)) || !aligned(bound, 4)) return AMOE_EALIGN;
+  const int CH = 16 / esize(dtype);
+  const long long rows = (long long)E * K;
+  const long long blocks = (rows * ((N + CH - 1) / CH) + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  const int vec = aligned(w, 16) && (N % CH == 0);
+  const int cvec = aligned(bound, 16) && (N % CH == 0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &clamp_weights_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<float*>(w), bound, rows, (int)K,
+                       (int)N, (int)cols, vec, cvec);
+  } else {
+    auto kf = &clamp_weights_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<uint16_t*>(w), bound, rows,
+                       (int)K, (int)N, (int)cols, vec, cvec);
   }
   return launch_rc();
 }

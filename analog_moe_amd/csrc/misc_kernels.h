@@ -92,17 +92,46 @@ __global__ __launch_bounds__(kThreads) void row_abs_max_kernel(const T* __restri
   if (row < rows && lane == 0) out[row] = m;
 }
 
-// cols == N: wmax[e, c] = max_k |w[e, k, c]|, one thread per column.
+// cols == N: wmax[e, c] = max_k |w[e, k, c]|.  Workgroup (column block, K slice, expert): a lane owns one 16-byte
+// chunk of columns, `width` lanes cover a row (or 64 chunks of it), the rest of the wave and the other three
+// waves take further rows; the slice's maxima meet in LDS and merge into the zero-filled output with an atomic
+// max on the bit pattern.
 template <typename T>
-__global__ __launch_bounds__(kThreads) void weight_col_abs_max_kernel(const T* __restrict__ w, int K, int N,
-                                                                       float* __restrict__ out) {
-  const int e = blockIdx.y;
-  const int c = blockIdx.x * kThreads + threadIdx.x;
-  if (c >= N) return;
-  const T* base = w + (long long)e * K * N + c;
-  float m = 0.f;
-  for (int k = 0; k < K; k++) m = fmaxf(m, fabsf(Elem<T>::load(base + (long long)k * N)));
-  out[(long long)e * N + c] = m;
+__global__ __launch_bounds__(kThreads) void weight_col_abs_max_kernel(const T* __restrict__ w, int K, int N, int width,
+                                                                       float* __restrict__ out, int vec) {
+  constexpr int CH = Elem<T>::kChunk;
+  __shared__ float red[kThreads][CH + 1];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rows_per_wave = 64 / width;
+  const int chunk = blockIdx.x * 64 + (lane % width);
+  const int row_in_block = wave * rows_per_wave + lane / width;
+  const int rows_per_block = 4 * rows_per_wave;
+  const int d = chunk * CH;
+  const int nv = N - d < CH ? N - d : CH;
+  const int e = blockIdx.z;
+  float m[CH];
+#pragma unroll
+  for (int q = 0; q < CH; q++) m[q] = 0.f;
+  if (nv > 0) {
+    const T* base = w + (long long)e * K * N + d;
+    for (int k = blockIdx.y * rows_per_block + row_in_block; k < K; k += gridDim.y * rows_per_block) {
+      float v[CH];
+      raw_unpack<T>(raw_load<T>(base + (long long)k * N, nv, vec != 0), v);
+#pragma unroll
+      for (int q = 0; q < CH; q++) m[q] = fmaxf(m[q], fabsf(v[q]));
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < CH; q++) red[tid][q] = m[q];
+  __syncthreads();
+  if (row_in_block == 0 && nv > 0) {
+    for (int r = 1; r < rows_per_block; r++) {
+      const int other = (r / rows_per_wave) * 64 + (r % rows_per_wave) * width + (lane % width);
+#pragma unroll
+      for (int q = 0; q < CH; q++) m[q] = fmaxf(m[q], red[other][q]);
+    }
+    for (int q = 0; q < nv; q++) atomicMax(reinterpret_cast<uint32_t*>(out) + (long long)e * N + d + q, as_u32(m[q]));
+  }
 }
 // cols == 1: wmax[e] = max |w[e]|.  grid (chunks, E): every workgroup reduces one slice and
 // merges with an atomic max on the bit pattern (non-negative floats order like integers), so the

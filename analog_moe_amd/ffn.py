@@ -33,6 +33,8 @@ class FFNConfig:
     input_min_percentage: float = 0.95
     noise_up: Optional[torch.Tensor] = None       # injected noise [n_tiles, T*k, F] (parity runs)
     noise_down: Optional[torch.Tensor] = None
+    wmax_up: Optional[torch.Tensor] = None        # max |W| behind noise and ADC when the weights passed in are
+    wmax_down: Optional[torch.Tensor] = None      # modified copies (fp32 [E, 1] or [E, N]); None: taken from them
 
 
 _SIDE_STREAMS = {}
@@ -48,7 +50,7 @@ def _side_stream(device: torch.device) -> "torch.cuda.Stream":
 
 CFG_FIELDS = ("inp_res", "bounds_up", "bounds_down", "out_bound", "out_res", "noise_std", "noise_seed",
               "noise_seed_dev", "noise_per_channel", "gradient_relative", "gradient_scale", "decay",
-              "input_min_percentage", "noise_up", "noise_down")
+              "input_min_percentage", "noise_up", "noise_down", "wmax_up", "wmax_down")
 
 
 def cfg_astuple(cfg: FFNConfig) -> tuple:
@@ -78,7 +80,9 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
     gen = cfg.noise_std > 0 and cfg.noise_up is None
     wu = wd = None
     main = torch.cuda.current_stream()
-    if cfg.out_bound > 0 or gen:
+    if cfg.wmax_up is not None:
+        wu, wd = cfg.wmax_up, cfg.wmax_down
+    elif cfg.out_bound > 0 or gen:
         # max |W| per expert only reads the weights: it runs next to the expert sort on a second stream
         side = _side_stream(x.device)
         side.wait_stream(main)
@@ -88,7 +92,7 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
         wu.record_stream(main)
         wd.record_stream(main)
     sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
-    if wu is not None:
+    if wu is not None and cfg.wmax_up is None:
         main.wait_stream(side)
     ir_up, ir_dn = ir_tables(input_range, E, cfg)
     common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,

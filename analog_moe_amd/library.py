@@ -10,6 +10,7 @@ so every group of calls the Python layer makes is one opaque operator with a fak
   amoe::offsets_from_sorted segment starts from sorted ids
   amoe::expert_std          per-expert std                    (cvmm.py:400-443)
   amoe::weight_abs_max      max |W| per expert / per channel  (moe_layer_aihwkit_lightning.py:476-489)
+  amoe::modify_weight       weight modifier of a forward      (moe_layer_aihwkit_lightning.py:313-382)
   amoe::cvmm_forward        everything CVMM.forward launches  (cvmm.py:701-769)
   amoe::cvmm_backward       everything CVMM.backward launches (cvmm.py:772-897)
   amoe::ffn_fwd / ffn_bwd   the fused expert feed-forward, with its autograd formula registered
@@ -122,6 +123,30 @@ def _(w, per_channel):
     return torch.empty((w.shape[0], w.shape[2] if per_channel else 1), dtype=torch.float32, device=w.device)
 
 
+@torch.library.custom_op(
+    "amoe::modify_weight", mutates_args=(),
+    schema="(Tensor w, bool per_channel, float n_states, float std_dev, Tensor? noise, bool round_noise, "
+           "int noise_seed, Tensor? noise_seed_dev) -> Tensor")
+def modify_weight(w, per_channel, n_states, std_dev, noise, round_noise, noise_seed, noise_seed_dev):
+    """The weight modifier of a training forward (moe_layer_aihwkit_lightning.py:313-382): a copy of
+    w [E, K, N] discretised to max |W| / n_states steps and / or with std_dev * max |W| * normal added."""
+    wmax = ops.weight_abs_max(w, per_channel)
+    return ops.modify_weight(w, wmax, n_states, std_dev, noise, round_noise, noise_seed, noise_seed_dev)
+
+
+@modify_weight.register_fake
+def _(w, per_channel, n_states, std_dev, noise, round_noise, noise_seed, noise_seed_dev):
+    return torch.empty(w.shape, dtype=w.dtype, device=w.device)
+
+
+def _modify_autograd(ctx, grad):
+    # straight-through quantiser, noise without gradient (moe_layer_aihwkit_lightning.py:362-377)
+    return (grad,) + (None,) * 7
+
+
+modify_weight.register_autograd(_modify_autograd)
+
+
 # --------------------------------------------------------------------------- CVMM forward / backward
 @torch.library.custom_op(
     "amoe::cvmm_forward", mutates_args=(),
@@ -203,7 +228,7 @@ def _(grad_output, x, keys, offsets, sel_index, out_index, gate, ir, z, bounds, 
 _CFG_SCHEMA = ("float inp_res, int[]? bounds_up, int[]? bounds_down, float out_bound, float out_res, "
                "float noise_std, int noise_seed, Tensor? noise_seed_dev, bool noise_per_channel, "
                "bool gradient_relative, float gradient_scale, float decay, float input_min_percentage, "
-               "Tensor? noise_up, Tensor? noise_down")
+               "Tensor? noise_up, Tensor? noise_down, Tensor? wmax_up, Tensor? wmax_down")
 _N_CFG = len(ffn.CFG_FIELDS)
 
 

@@ -28,6 +28,7 @@ from torch import Tensor, nn
 from .config import (AIHWKITTorchInferenceRPUConfig, TorchInferenceRPUConfig, enum_name, kernel_inp_res)
 from .cvmm import CVMM, AnalogExt, CVMMSel, cvmm_prepare_sel2, cvmm_std
 from . import library  # noqa: F401  (registers the amoe:: operators)
+from . import ops
 from .ffn import FFNConfig, moe_ffn
 
 
@@ -242,7 +243,9 @@ class AnalogLinear(nn.Module):
         modified = w
         if (self.training or self.rpu_config.modifier.enable_during_test) and \
                 enum_name(self.rpu_config.modifier.type) not in ("NONE", "COPY"):
-            modified = AnalogSigmaMoELayer.modify_weight(w.clone(), self.rpu_config.modifier)
+            modified = AnalogSigmaMoELayer.modify_weight(
+                w, self.rpu_config.modifier, injected=self.noise_mode == "injected", seed_dev=self.noise_counter,
+                seed=None if self.noise_mode == "injected" else self._seed() ^ _MODIFIER_ROUTER_SEED)
         ext = AnalogExt(offsets=sel.offsets, bounds=self.bounds,
                         out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
                         out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
@@ -263,13 +266,54 @@ class AnalogLinear(nn.Module):
     @torch.no_grad()
     def clip_weights(self) -> None:
         kind = enum_name(self.rpu_config.clip.type)
-        if kind in ("LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL"):
-            dims = None if kind == "LAYER_GAUSSIAN" else 1
-            bound = self.rpu_config.clip.sigma * (self.weight.std() if dims is None else self.weight.std(1, keepdim=True))
-            self.weight.data = torch.minimum(torch.maximum(self.weight.data, -bound), bound)
+        out, inp = self.weight.shape
+        if kind == "LAYER_GAUSSIAN":                  # one bound for the whole matrix
+            _gaussian_clip_(self.weight.data.view(1, out, inp), self.rpu_config.clip.sigma, False)
+        elif kind == "LAYER_GAUSSIAN_PER_CHANNEL":    # one per output channel = per row of weight [out, in]
+            _gaussian_clip_(self.weight.data.view(out, inp, 1), self.rpu_config.clip.sigma, False)
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, tiles={self.n_tiles}"
+
+
+_LIGHTNING_MODIFIERS = ("DISCRETIZE", "DISCRETIZE_PER_CHANNEL", "ADD_NORMAL", "ADD_NORMAL_PER_CHANNEL",
+                        "DISCRETIZE_ADD_NORMAL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL")
+_MODIFIER_DOWN_SEED = 0x5851F42D4C957F2D     # keep the draws for the weight tensors of a layer apart
+_MODIFIER_ROUTER_SEED = 0x2545F4914F6CDD1D
+_STATIC_MODIFIER_CALLS = [0]
+
+
+def _need_device(w: Tensor, what: str) -> None:
+    if not (w.is_cuda or w.is_meta):
+        raise MoEConifgError(f"{what} on CPU tensors. This package runs on the GPU only.")
+
+
+def _modify_on_device(w: Tensor, per_channel: bool, n_states: float, std_dev: float, round_noise: bool,
+                      seed: Optional[int], seed_dev: Optional[Tensor], injected: bool) -> Tensor:
+    """One pass of the weight-modifier kernel over w [E, K, N] (``amoe::modify_weight``)."""
+    _need_device(w, "Weight modifier")
+    noise = None
+    if std_dev > 0 and injected:
+        with torch.no_grad():
+            noise = torch.randn_like(w) if round_noise else torch.randn(w.shape, device=w.device)
+    elif std_dev > 0 and seed is None:
+        # a call without a layer behind it (the reference's static method): torch's seed and a call count
+        _STATIC_MODIFIER_CALLS[0] += 1
+        seed = (torch.initial_seed() * 0x9E3779B97F4A7C15 + _STATIC_MODIFIER_CALLS[0] * 0xD1B54A32D192ED03) & (2 ** 63 - 1)
+    return torch.ops.amoe.modify_weight(w, per_channel, n_states, std_dev, noise, round_noise, int(seed or 0),
+                                        seed_dev if std_dev > 0 and noise is None else None)
+
+
+def _gaussian_clip_(w: Tensor, sigma: float, per_channel: bool, max_bound: float = -1.0) -> None:
+    """w = clamp(w, +-sigma * std) in place, std per expert or per channel, rounded as ``sigma * w.std(...)``
+    rounds (moe_layer_aihwkit_lightning.py:529-541); max_bound > 0 caps the bound (moe_layer_aihwkit.py:332-333)."""
+    _need_device(w, "Weight clipping")
+    if w.is_meta:
+        return
+    bound = sigma * ops.weight_std(w, per_channel).to(w.dtype)
+    if max_bound > 0:
+        bound = bound.clamp(max=max_bound)
+    ops.clamp_weights_(w, bound)
 
 
 def load_state_dict_pre_hook(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
@@ -389,36 +433,39 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     def _modifier_on(self) -> bool:
         return enum_name(self.rpu_config.modifier.type) != "NONE"
 
-    def _modified(self, weights: Tensor) -> Tensor:
-        return self.modify_weight(weights.clone(), self.rpu_config.modifier)
+    def _modified(self, weights: Tensor, is_down: bool = False) -> Tensor:
+        return self.modify_weight(weights, self.rpu_config.modifier, **self._modifier_draw(is_down))
 
     def _row_abs_max_on(self) -> bool:
         """Whether CVMM will scale every input row by its abs-max (cvmm.py:727-739)."""
         return self.input_range is None
 
+    def _modifier_draw(self, is_down: bool) -> dict:
+        """Where the modifier's normals come from: the layer's seed (and its device counter) for the kernel's
+        generator, or -- ``noise_mode="injected"`` -- torch's own stream, as the reference draws them."""
+        if self.noise_mode == "injected":
+            return dict(injected=True)
+        seed = self._noise_seed() ^ (_MODIFIER_DOWN_SEED if is_down else 0)
+        return dict(seed=seed, seed_dev=self.noise_counter)
+
     # -- weight modifier / clipping (moe_layer_aihwkit_lightning.py:313-382, 509-543) -----------------
     @staticmethod
-    def modify_weight(inp_weight: Tensor, modifier) -> Tensor:
+    def modify_weight(inp_weight: Tensor, modifier, *, seed: Optional[int] = None, seed_dev: Optional[Tensor] = None,
+                      injected: bool = False) -> Tensor:
+        """A modified copy of ``inp_weight`` [E, K, N] (one kernel pass; the reference clones and modifies in
+        place).  The gradient of the result reaches ``inp_weight`` unchanged."""
         kind = enum_name(modifier.type)
         if kind == "NONE":
             return inp_weight
+        if kind not in _LIGHTNING_MODIFIERS:
+            raise MoEConifgError(f"Weight modifier {modifier} not supported")
         # per-channel max |W| for the two discretising per-channel types only: the reference's list
         # (moe_layer_aihwkit_lightning.py:333-337) names DISCRETIZE_ADD_NORMAL_PER_CHANNEL twice and leaves
         # ADD_NORMAL_PER_CHANNEL out, so that type scales its noise by the per-expert maximum -- kept as it is
-        if kind in ("DISCRETIZE_PER_CHANNEL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL"):
-            wmax = inp_weight.abs().amax(1, keepdim=True)
-        else:
-            wmax = inp_weight.reshape(inp_weight.size(0), -1).abs().amax(-1).view(-1, 1, 1)
-        if kind.startswith("DISCRETIZE"):
-            n_states = max(modifier.res, 1 / modifier.res)
-            res = wmax / n_states
-            q = torch.round(inp_weight / res) * res
-            inp_weight = inp_weight + (q - inp_weight).detach()        # straight-through quantiser
-        if "ADD_NORMAL" in kind:
-            with torch.no_grad():
-                noise = modifier.std_dev * wmax * torch.randn_like(inp_weight)
-            inp_weight = inp_weight + noise
-        return inp_weight
+        per_channel = kind in ("DISCRETIZE_PER_CHANNEL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL")
+        n_states = float(max(modifier.res, 1 / modifier.res)) if kind.startswith("DISCRETIZE") else 0.0
+        std_dev = float(modifier.std_dev) if "ADD_NORMAL" in kind else 0.0
+        return _modify_on_device(inp_weight, per_channel, n_states, std_dev, True, seed, seed_dev, injected)
 
     def post_update_step(self) -> None:
         if hasattr(self.rpu_config, "clip") and enum_name(self.rpu_config.clip.type) != "NONE":
@@ -435,10 +482,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         assert sigma > 0, "Clip sigma must be greater than 0"
         if kind not in ("LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL"):
             raise ValueError(f"Unknown clip type {self.rpu_config.clip.type}")
-        dims = (1, 2) if kind == "LAYER_GAUSSIAN" else 1
         for w in (self.keys, self.values):
-            bound = sigma * w.std(dims, keepdim=True)
-            w.data = torch.minimum(torch.maximum(w.data, -bound), bound)
+            _gaussian_clip_(w.data, sigma, kind == "LAYER_GAUSSIAN_PER_CHANNEL")
 
     # -- the analog matmul ------------------------------------------------------------------------------
     def _update_input_range_from_data(self, inputs: Tensor, sel_indices: CVMMSel, ir_idx: int) -> None:
@@ -512,7 +557,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         inp_res = -1.0 if perfect else kernel_inp_res(fwd.inp_res)
         modified = weights
         if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
-            modified = self._modified(weights)
+            modified = self._modified(weights, is_down=not is_up)
         ext = AnalogExt(offsets=sel_indices.offsets, bounds=bounds,
                         out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
                         out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
@@ -537,7 +582,7 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
     # -- fused path ---------------------------------------------------------------------------------------
     def _fusable(self) -> bool:
         return (self.activation is F.relu and self.bias is None and self.dropout == 0 and
-                self.input_range is not None and not self._row_abs_max_on() and not self._modifier_on() and
+                self.input_range is not None and not self._row_abs_max_on() and
                 not (self.training and self._init_from_data_pending()))
 
     def forward_selected(self, x: Tensor, sel_val: Tensor, sel_idx: Tensor) -> Tensor:
@@ -568,8 +613,16 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             ntd = 1 if self.bounds_down is None else len(self.bounds_down) - 1
             cfg.noise_up = torch.randn(ntu, M, self.expert_size, device=x.device) * fwd.out_noise * wu[flat]
             cfg.noise_down = torch.randn(ntd, M, self.v_dim, device=x.device) * fwd.out_noise * wd[flat]
+        keys, values = self.keys, self.values
+        if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
+            # the output noise and the ADC keep following the max |W| of the unmodified weights
+            # (moe_layer_aihwkit_lightning.py:458-489)
+            if noisy or cfg.out_bound > 0:
+                cfg.wmax_up = torch.ops.amoe.weight_abs_max(keys.detach(), cfg.noise_per_channel)
+                cfg.wmax_down = torch.ops.amoe.weight_abs_max(values.detach(), cfg.noise_per_channel)
+            keys, values = self._modified(keys, is_down=False), self._modified(values, is_down=True)
         lead = x.shape[:-1]
-        y = moe_ffn(x.reshape(-1, x.shape[-1]), self.keys.to(x.dtype), self.values.to(x.dtype),
+        y = moe_ffn(x.reshape(-1, x.shape[-1]), keys.to(x.dtype), values.to(x.dtype),
                     self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
                     sel_idx.reshape(-1, self.n_heads), cfg)
         if cfg.noise_seed_dev is not None:
@@ -640,16 +693,18 @@ class AnalogSigmaMoELayerAIHWKIT(AnalogSigmaMoELayer):
     def _modifier_on(self) -> bool:
         return enum_name(self.rpu_config.modifier.type) not in ("NONE", "COPY")
 
-    def _modified(self, weights: Tensor) -> Tensor:
-        return self.modify_weight(weights, self.rpu_config.modifier, self.rpu_config.remap.type)
+    def _modified(self, weights: Tensor, is_down: bool = False) -> Tensor:
+        return self.modify_weight(weights, self.rpu_config.modifier, self.rpu_config.remap.type,
+                                  **self._modifier_draw(is_down))
 
     def _row_abs_max_on(self) -> bool:
         fwd = self.rpu_config.forward
         return not fwd.is_perfect and enum_name(fwd.noise_management) == "ABS_MAX"
 
     @staticmethod
-    def modify_weight(inp_weight: Tensor, modifier, remap_type=None) -> Tensor:
-        """moe_layer_aihwkit.py:144-196."""
+    def modify_weight(inp_weight: Tensor, modifier, remap_type=None, *, seed: Optional[int] = None,
+                      seed_dev: Optional[Tensor] = None, injected: bool = False) -> Tensor:
+        """moe_layer_aihwkit.py:144-196: ADD_NORMAL only, max |W| by remap type, fp32 normals."""
         if getattr(modifier, "per_batch_sample", False):
             raise MoEConifgError("per_batch_sample not implemented")
         kind = enum_name(modifier.type)
@@ -658,19 +713,14 @@ class AnalogSigmaMoELayerAIHWKIT(AnalogSigmaMoELayer):
         if kind == "MULT_NORMAL":
             raise MoEConifgError("MULT_NORMAL not implemented")
         remap = enum_name(remap_type)
-        if remap == "CHANNELWISE_SYMMETRIC":
-            wmax = inp_weight.abs().amax(1).unsqueeze(1)                        # [E, 1, N]
-        elif remap == "LAYERWISE_SYMMETRIC":
-            wmax = inp_weight.reshape(inp_weight.size(0), -1).abs().amax(-1).view(-1, 1, 1)
-        else:
+        if remap not in ("CHANNELWISE_SYMMETRIC", "LAYERWISE_SYMMETRIC"):
             raise MoEConifgError(f"Weight remap type {remap_type} not supported")
         if kind == "DISCRETIZE":
             raise MoEConifgError("DISCRETIZE not implemented")
         if kind != "ADD_NORMAL":
             raise MoEConifgError(f"Weight modifier {modifier} not supported")
-        with torch.no_grad():
-            noise = modifier.std_dev * wmax * torch.randn(inp_weight.shape, device=inp_weight.device)
-        return inp_weight.clone() + noise.to(inp_weight.dtype)
+        return _modify_on_device(inp_weight, remap == "CHANNELWISE_SYMMETRIC", 0.0, float(modifier.std_dev), False,
+                                 seed, seed_dev, injected)
 
     def post_update_step(self) -> None:
         if hasattr(self.rpu_config, "clip") and enum_name(self.rpu_config.clip.type) != "NONE":
@@ -683,13 +733,12 @@ class AnalogSigmaMoELayerAIHWKIT(AnalogSigmaMoELayer):
         kind = enum_name(clip.type)
         if kind == "FIXED_VALUE":
             for w in (self.keys, self.values):
-                w.data = torch.clamp(w, -clip.fixed_value, clip.fixed_value)
+                _need_device(w, "Weight clipping")
+                if not w.is_meta:
+                    ops.clamp_weights_(w.data, torch.full((w.shape[0],), float(clip.fixed_value), device=w.device))
         elif kind == "LAYER_GAUSSIAN":
             for w in (self.keys, self.values):
-                alpha = w.std((1, 2), keepdim=True) * clip.sigma
-                if clip.fixed_value > 0:
-                    alpha = alpha.clamp(max=clip.fixed_value)
-                w.data = torch.minimum(torch.maximum(w.data, -alpha), alpha)
+                _gaussian_clip_(w.data, clip.sigma, False, max_bound=clip.fixed_value)
         elif kind == "AVERAGE_CHANNEL_MAX":
             raise NotImplementedError("AVERAGE_CHANNEL_MAX not implemented")
         else:

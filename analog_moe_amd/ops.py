@@ -232,3 +232,44 @@ def expert_std(x: torch.Tensor, in_index: torch.Tensor, offsets: torch.Tensor, n
     out = torch.empty(n_experts, dtype=torch.float32, device=x2.device)
     raw.expert_std(get_lib(), _stream(x2), x2, _i32c(in_index), offsets, n_experts, out)
     return out
+
+
+# ------------------------------------------------------------------------------ weight modifier / clip
+def modify_weight(w: torch.Tensor, wmax: torch.Tensor, n_states: float = 0.0, std_dev: float = 0.0,
+                  noise: Optional[torch.Tensor] = None, round_noise: bool = True, noise_seed: int = 0,
+                  noise_seed_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Modified copy of w [E, K, N]: discretised to multiples of wmax / n_states (n_states > 0), plus
+    std_dev * wmax * normal (std_dev > 0).  wmax: fp32 [E, 1] or [E, N] as ``weight_abs_max`` returns it."""
+    _need_gpu(w, wmax, noise, noise_seed_dev)
+    wc = w.detach().contiguous()
+    out = torch.empty_like(wc)
+    raw.modify_weight(get_lib(), _stream(wc), wc, _f32c(wmax), n_states, std_dev, _f32c(noise), round_noise,
+                      noise_seed, noise_seed_dev, out)
+    return out
+
+
+def weight_std(w: torch.Tensor, per_channel: bool) -> torch.Tensor:
+    """Unbiased std of w [E, K, N] over (K, N) -> [E, 1, 1] or over K -> [E, 1, N], fp32."""
+    _need_gpu(w)
+    lib = get_lib()
+    wc = w.detach().contiguous()
+    E, K, N = wc.shape
+    cols = N if per_channel else 1
+    out = torch.empty((E, 1, cols), dtype=torch.float32, device=wc.device)
+    nbytes = raw.weight_std_workspace_bytes(lib, E, K, N, cols)
+    ws = torch.empty(nbytes // 8, dtype=torch.float64, device=wc.device) if nbytes else None
+    raw.weight_std(lib, _stream(wc), wc, cols, out, ws)
+    return out
+
+
+def clamp_weights_(w: torch.Tensor, bound: torch.Tensor) -> torch.Tensor:
+    """w = clamp(w, -bound, bound) in place; bound broadcasts as [E, 1, 1] or [E, 1, N]."""
+    _need_gpu(w, bound)
+    if not w.is_contiguous():
+        raise ValueError("clamp_weights_ works in place on a contiguous tensor")
+    E, K, N = w.shape
+    cols = bound.numel() // E
+    if cols not in (1, N) or bound.numel() != E * cols:
+        raise ValueError("bound must hold one value per expert or per expert and channel")
+    raw.clamp_weights(get_lib(), _stream(w), w.detach(), _f32c(bound), cols)
+    return w

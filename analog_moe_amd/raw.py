@@ -227,3 +227,44 @@ def expert_std(lib, stream, x, in_index, offsets, E: int, out):
     check(lib, lib.amoe_expert_std(dtype_code(x), _p(x), x.stride(0), x.shape[1], _p(_i32(in_index, "in_index")),
                                    _p(_i32(offsets, "offsets")), E, _p(_f32(out, "out")), stream),
           "amoe_expert_std")
+
+
+def modify_weight(lib, stream, w, wmax, n_states: float, std_dev: float, noise, round_noise: bool, noise_seed: int,
+                  noise_seed_dev, out):
+    if not w.is_contiguous() or not out.is_contiguous() or out.shape != w.shape or out.dtype != w.dtype:
+        raise ValueError("w and out must be contiguous tensors of one shape and dtype")
+    E, K, N = w.shape
+    cols = wmax.numel() // E
+    if wmax.numel() != E * cols or cols not in (1, N):
+        raise ValueError("wmax must be [E] or [E, N]")
+    if noise is not None and noise.numel() != w.numel():
+        raise ValueError("noise must have one value per weight")
+    if noise_seed_dev is not None and (noise_seed_dev.dtype != torch.int64 or noise_seed_dev.numel() != 1):
+        raise ValueError("noise_seed_dev must be one int64 word")
+    check(lib, lib.amoe_modify_weight(dtype_code(w), _p(w), E, K, N, _p(_f32(wmax, "wmax")), cols, float(n_states),
+                                      float(std_dev), _p(_f32(noise, "noise")), int(bool(round_noise)),
+                                      int(noise_seed) & 0xFFFFFFFFFFFFFFFF, _p(noise_seed_dev), _p(out), stream),
+          "amoe_modify_weight")
+
+
+def weight_std_workspace_bytes(lib, E: int, K: int, N: int, cols: int) -> int:
+    return lib.amoe_weight_std_workspace(E, K, N, cols)
+
+
+def weight_std(lib, stream, w, cols: int, out, workspace):
+    if not w.is_contiguous():
+        raise ValueError("w must be contiguous")
+    E, K, N = w.shape
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib, lib.amoe_weight_std(dtype_code(w), _p(w), E, K, N, cols, _p(_f32(out, "std")), _p(workspace), nbytes,
+                                   stream), "amoe_weight_std")
+
+
+def clamp_weights(lib, stream, w, bound, cols: int):
+    if not w.is_contiguous():
+        raise ValueError("w must be contiguous")
+    E, K, N = w.shape
+    if bound.numel() != E * cols:
+        raise ValueError("bound must be [E] or [E, N]")
+    check(lib, lib.amoe_clamp_weights(dtype_code(w), _p(w), E, K, N, _p(_f32(bound, "bound")), cols, stream),
+          "amoe_clamp_weights")

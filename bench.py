@@ -179,6 +179,9 @@ def main():
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=1024)
+    ap.add_argument("--modifier", default="none",
+                    help="weight modifier type of the training forward (e.g. add_normal_per_channel, "
+                         "discretize_add_normal_per_channel); not part of the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 256 MiB device copy first (reference reading for HBM counters)")
@@ -210,6 +213,9 @@ def main():
     rpu.pre_post.input_range.learn_input_range = True
     rpu.pre_post.input_range.init_value = 3.0
     rpu.pre_post.input_range.decay = 0.01
+    if args.modifier.lower() != "none":
+        rpu.modifier.type = cfgmod.WeightModifierType[args.modifier.upper()]
+        rpu.modifier.std_dev, rpu.modifier.res = 0.02, 2 ** 8 - 2
     torch.manual_seed(0)
     layer = AnalogSigmaMoELayer(rpu, d_model=D, n_experts=E, expert_size=F, k=k).to(dev).to(tdt)
     layer.train()
@@ -325,7 +331,9 @@ def main():
         "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["name"], "tokens": T, "d_model": D, "n_experts": E, "expert_size": F,
                    "top_k": k, "analog": "learned input range 3.0, 8-bit DAC, 8-bit ADC (out_bound 12), "
-                   f"output noise {cfg['noise']} x max|W| drawn in-kernel, max_input_size {cfg['mis']}"},
+                   f"output noise {cfg['noise']} x max|W| drawn in-kernel, max_input_size {cfg['mis']}"
+                   + ("" if args.modifier.lower() == "none" else f", weight modifier {args.modifier.lower()} "
+                      "(std_dev 0.02, 254 states)")},
         "tflops": flops_step / (ms * 1e-3) / 1e12,
         "pct_of_mfma_peak": 100.0 * flops_step / (ms * 1e-3) / peak,
         "roofline": {"bound": "mfma", "kernel": dom,

@@ -240,6 +240,39 @@ int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K,
                     const int32_t* in_index, const int32_t* offsets, int32_t E,
                     float* out, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Weight modifier of a training forward: out [E, K, N] = modified copy of w
+ * (AnalogSigmaMoELayerAIHWKITLightning.modify_weight, moe_layer_aihwkit_lightning.py:313-382;
+ * the ADD_NORMAL case of moe_layer_aihwkit.py:144-196).
+ *   n_states > 0:  res = wmax * (1 / n_states);  w = round(w / res) * res  (:346-363; torch's GPU
+ *                  kernels divide a tensor by a host scalar through the fp32 reciprocal)
+ *   std_dev  > 0:  w += std_dev * wmax * z,  z standard normal             (:364-379)
+ * wmax is the assumed max |W|: [E] (wmax_cols == 1) or [E, N] (wmax_cols == N), fp32, as
+ * amoe_weight_abs_max writes it (:333-344).  z comes from `noise` (fp32 [E, K, N]) when given,
+ * else from the counter-based generator keyed by noise_seed (+ *noise_seed_dev) and the
+ * element's position.  For bf16 every intermediate is rounded where the reference's tensor
+ * expression rounds it; round_noise != 0 also rounds z to the weights' type first (randn_like
+ * of the weights, :366) and 0 leaves it fp32 (moe_layer_aihwkit.py:188-194).
+ * The gradient of the modified weights is passed to w unchanged by the caller. */
+int amoe_modify_weight(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N,
+                       const float* wmax, int32_t wmax_cols, float n_states, float std_dev,
+                       const float* noise, int32_t round_noise, uint64_t noise_seed,
+                       const uint64_t* noise_seed_dev, void* out, void* stream);
+
+/* Unbiased standard deviation of the weights per expert (cols == 1: std_out [E]) or per
+ * channel (cols == N: std_out [E, N]): the std((1, 2)) / std(1) of clip_weights
+ * (moe_layer_aihwkit_lightning.py:529-534; moe_layer_aihwkit.py:327-331).  fp32 result.
+ * workspace: amoe_weight_std_workspace bytes, 8-byte aligned (partial sums in fp64, added in a
+ * fixed order). */
+size_t amoe_weight_std_workspace(int32_t E, int32_t K, int32_t N, int32_t cols);
+int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols,
+                    float* std_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* w = clamp(w, -bound, +bound) in place, bound [E] (cols == 1) or [E, N] (cols == N), fp32
+ * (moe_layer_aihwkit_lightning.py:535-541; moe_layer_aihwkit.py:321-335). */
+int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N,
+                       const float* bound, int32_t cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -132,11 +132,28 @@ def test_companions(emu_ops):
     assert torch.equal(emu_ops.row_abs_max(x), x.abs().amax(-1))
     assert torch.equal(emu_ops.weight_abs_max(pr["keys"], False), pr["keys"].abs().amax((1, 2)).reshape(5, 1))
     assert torch.equal(emu_ops.weight_abs_max(pr["keys"], True), pr["keys"].abs().amax(1))
+    util.check_weight_abs_max(emu_ops)
     s = emu_ops.prepare_sel(pr["idx"].clamp(max=3), 5, 2)
     std = emu_ops.expert_std(x, s[2], s[3], 5)
     want = O.expert_std(x.numpy(), s[2].numpy(), s[0].numpy(), 5)
     np.testing.assert_allclose(std.numpy()[:4], want[:4], rtol=1e-5)
     assert not (std[4] > 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", util.MODIFIER_KINDS)
+def test_weight_modifier_matches_oracle(emu_ops, kind, dtype):
+    util.check_modify_weight(emu_ops, kind, dtype)
+    util.check_modify_weight(emu_ops, kind, dtype, E=2, K=9, N=13)          # ragged rows: the scalar paths
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_weight_std_and_clamp_match_oracle(emu_ops, per_channel, dtype):
+    util.check_weight_clip(emu_ops, per_channel, dtype)
+    util.check_weight_clip(emu_ops, per_channel, dtype, E=2, K=33, N=7)
+    if not per_channel:
+        util.check_weight_clip(emu_ops, per_channel, dtype, E=2, K=300, N=200)   # several slices per expert
 
 
 def test_transposed_weight_view(emu_ops):

@@ -85,28 +85,23 @@ def test_inp_res_mapping_and_weight_modifier():
     assert cfg.kernel_inp_res(2 ** 8 - 2) == pytest.approx(1 / 127)
     assert cfg.kernel_inp_res(1 / (2 ** 8 - 2)) == pytest.approx(1 / 127)
     assert cfg.kernel_inp_res(-1) == -1
+    # the modifier and the clip are kernels: host tensors are refused, nothing is computed on the CPU
     w = torch.randn(3, 8, 5)
     m = cfg.WeightModifierParameter(type=cfg.WeightModifierType.DISCRETIZE_PER_CHANNEL, res=2 ** 4 - 2)
-    q = AnalogSigmaMoELayer.modify_weight(w.clone(), m)
-    step = w.abs().amax(1, keepdim=True) / 14
-    assert torch.allclose(q / step, torch.round(q / step), atol=1e-4)
-    m2 = cfg.WeightModifierParameter(type=cfg.WeightModifierType.ADD_NORMAL, std_dev=0.1)
-    assert not torch.equal(AnalogSigmaMoELayer.modify_weight(w.clone(), m2), w)
-    # ADD_NORMAL_PER_CHANNEL scales its noise by the per-expert maximum, as the reference's type list makes it
-    # (moe_layer_aihwkit_lightning.py:333-337): a quiet channel gets the same noise as a loud one
-    torch.manual_seed(0)
-    wq = torch.randn(2, 256, 6)
-    wq[:, :, 0] *= 20
-    m3 = cfg.WeightModifierParameter(type=cfg.WeightModifierType.ADD_NORMAL_PER_CHANNEL, std_dev=0.1)
-    d = AnalogSigmaMoELayer.modify_weight(wq.clone(), m3) - wq
-    assert d[:, :, 0].std() == pytest.approx(d[:, :, 1:].std().item(), rel=0.2)
-    assert d[0].std() == pytest.approx(0.1 * wq[0].abs().max().item(), rel=0.15)
+    with pytest.raises(MoEConifgError, match="GPU only"):
+        AnalogSigmaMoELayer.modify_weight(w, m)
+    assert AnalogSigmaMoELayer.modify_weight(w, cfg.WeightModifierParameter()) is w          # NONE: untouched
+    with pytest.raises(MoEConifgError, match="not supported"):
+        AnalogSigmaMoELayer.modify_weight(w, cfg.WeightModifierParameter(type=cfg.WeightModifierType.MULT_NORMAL))
+    q = AnalogSigmaMoELayer.modify_weight(w.to("meta"), m)                                    # shape inference only
+    assert q.is_meta and q.shape == w.shape
     layer = AnalogSigmaMoELayer(_rpu(), d_model=8, n_experts=3, expert_size=5, k=1)
     layer.rpu_config.clip.type = cfg.WeightClipType.LAYER_GAUSSIAN
     layer.rpu_config.clip.sigma = 1.0
-    before = layer.keys.data.abs().max().item()
+    with pytest.raises(MoEConifgError, match="GPU only"):
+        layer.post_update_step()
+    layer.rpu_config.clip.type = cfg.WeightClipType.NONE
     layer.post_update_step()
-    assert layer.keys.data.abs().max().item() < before
 
 
 def _aihwkit_rpu(**fw):
@@ -153,28 +148,22 @@ def test_aihwkit_flavour_modifier_and_clip():
     assert mod(w, M(type=cfg.WeightModifierType.NONE), R.LAYERWISE_SYMMETRIC) is w
     assert mod(w, M(type=cfg.WeightModifierType.COPY), R.LAYERWISE_SYMMETRIC) is w
     add = M(type=cfg.WeightModifierType.ADD_NORMAL, std_dev=0.1)
-    d_layer = mod(w, add, R.LAYERWISE_SYMMETRIC) - w
-    d_chan = mod(w, add, R.CHANNELWISE_SYMMETRIC) - w
-    wmax_layer = w.reshape(3, -1).abs().amax(-1)
-    assert torch.allclose(d_layer.reshape(3, -1).std(-1), 0.1 * wmax_layer, rtol=0.1)
-    assert torch.allclose(d_chan.std(1), 0.1 * w.abs().amax(1), rtol=0.35)   # 64 samples per channel
-    assert d_chan[:, :, 0].std() > 3 * d_chan[:, :, 1:].std()
     for bad in (M(type=cfg.WeightModifierType.MULT_NORMAL), M(type=cfg.WeightModifierType.DISCRETIZE),
                 M(type=cfg.WeightModifierType.ADD_NORMAL, per_batch_sample=True)):
         with pytest.raises(MoEConifgError):
             mod(w, bad, R.LAYERWISE_SYMMETRIC)
     with pytest.raises(MoEConifgError):
         mod(w, add, R.NONE)
+    with pytest.raises(MoEConifgError, match="GPU only"):
+        mod(w, add, R.LAYERWISE_SYMMETRIC)
     layer = AnalogSigmaMoELayerAIHWKIT(_aihwkit_rpu(), d_model=8, n_experts=3, expert_size=5, k=1)
     layer.rpu_config.clip = cfg.WeightClipParameter(type=cfg.WeightClipType.FIXED_VALUE, fixed_value=0.05)
-    layer.post_update_step()
-    assert layer.keys.data.abs().max().item() <= 0.05 + 1e-7 and layer.values.data.abs().max().item() <= 0.05 + 1e-7
-    layer.reset_parameters()
-    std = layer.keys.data.std((1, 2), keepdim=True)
-    layer.clip_weights(cfg.WeightClipParameter(type=cfg.WeightClipType.LAYER_GAUSSIAN, sigma=1.0))
-    assert bool((layer.keys.data.abs() <= std * (1 + 1e-6)).all())
+    with pytest.raises(MoEConifgError, match="GPU only"):
+        layer.post_update_step()
     with pytest.raises(NotImplementedError):
         layer.clip_weights(cfg.WeightClipParameter(type=cfg.WeightClipType.AVERAGE_CHANNEL_MAX))
+    with pytest.raises(MoEConifgError):
+        layer.clip_weights(cfg.WeightClipParameter(type=cfg.WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL))
 
 
 def test_aihwkit_flavour_state_dict_carries_the_config():

@@ -372,3 +372,94 @@ def test_per_expert_torch_layer_agrees_with_oracle(quant):
     np.testing.assert_allclose(r.grad_x, xs.grad.numpy(), **tol)
     np.testing.assert_allclose(r.grad_gate, gs.grad.numpy(), **tol)
     np.testing.assert_allclose(r.grad_ir, irs.grad.numpy(), rtol=1e-3, atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------- weight modifier / clip
+from oracle import weights_oracle as WO   # noqa: E402
+from tests import util   # noqa: E402
+
+
+def _torch_modify(w, kind, res, std_dev, z):
+    """moe_layer_aihwkit_lightning.py:331-381 as tensor operations evaluated by torch on the CPU, with the
+    quantiser written as round(w / res) * res."""
+    if kind in WO.PER_CHANNEL_WMAX:
+        wmax = w.abs().amax(1).unsqueeze(1)
+    else:
+        wmax = w.view(w.size(0), -1).abs().amax(-1).view(-1, 1, 1)
+    if kind.startswith("DISCRETIZE"):
+        n_states = max(res, 1 / res)
+        step = wmax * torch.tensor(1.0, dtype=torch.float32).div(n_states).item()   # GPU kernels use the reciprocal
+        w = torch.round(w / step) * step
+    if "ADD_NORMAL" in kind:
+        w = w + std_dev * wmax * z
+    return w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", util.MODIFIER_KINDS)
+def test_modify_weight_oracle_matches_torch_expression(kind, dtype):
+    w = util.modifier_weights(1, 3, 30, 10, dtype)
+    z = torch.randn(3, 30, 10, generator=torch.Generator().manual_seed(2)).to(dtype)
+    want = _torch_modify(w, kind, 14.0, 0.07, z)
+    got = WO.modify_weight(util.np32(w), kind, 14.0, 0.07, util.np32(z), "bf16" if dtype == torch.bfloat16 else "f32")
+    assert np.array_equal(got, util.np32(want))
+
+
+def test_modify_weight_oracle_wmax_follows_the_reference_type_list():
+    """ADD_NORMAL_PER_CHANNEL is missing from the per-channel list (moe_layer_aihwkit_lightning.py:333-337): its
+    noise is scaled by the per-expert maximum, so a quiet channel gets the noise of the loud one."""
+    w = util.np32(util.modifier_weights(1, 2, 64, 6))
+    z = np.ones_like(w)
+    d = WO.modify_weight(w, "ADD_NORMAL_PER_CHANNEL", std_dev=0.1, z=z) - w
+    np.testing.assert_allclose(d, np.broadcast_to(0.1 * np.abs(w).max(axis=(1, 2), keepdims=True), w.shape), rtol=1e-5)
+    d = WO.modify_weight(w, "DISCRETIZE_ADD_NORMAL_PER_CHANNEL", res=1e6, std_dev=0.1, z=z) - w
+    np.testing.assert_allclose(d, np.broadcast_to(0.1 * np.abs(w).max(axis=1, keepdims=True), w.shape), rtol=1e-3,
+                               atol=1e-6)
+    assert WO.modify_weight(w, "NONE") is not None and np.array_equal(WO.modify_weight(w, "NONE"), w)
+
+
+@pytest.mark.parametrize("kind", ["DISCRETIZE", "DISCRETIZE_PER_CHANNEL"])
+def test_discretize_oracle_is_a_uniform_quantiser(kind):
+    """What any quantiser to n_states steps of max |W| must satisfy, whatever its rounding of ties."""
+    w = util.np32(util.modifier_weights(4, 3, 50, 8))
+    res = 2 ** 4 - 2
+    q = WO.modify_weight(w, kind, res)
+    wmax = WO.assumed_wmax(w, kind in WO.PER_CHANNEL_WMAX)
+    step = wmax / res
+    codes = q / step
+    np.testing.assert_allclose(codes, np.rint(codes), atol=1e-4)            # multiples of the step
+    assert np.abs(codes).max() <= res + 1e-4 and np.abs(codes).max() >= res - 1e-4   # max |W| is the last level
+    assert (np.abs(q - w) <= step / 2 * (1 + 1e-5)).all()                      # nearest level
+    assert np.array_equal(WO.modify_weight(q, kind, res, wmax=wmax), q)        # idempotent
+    assert np.array_equal(WO.modify_weight(w, kind, 1 / res), q)               # res and 1 / res mean the same
+    assert len(np.unique(np.rint(codes[0]))) <= 2 * res + 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL"])
+def test_clip_oracle_matches_numpy_and_torch(kind, dtype):
+    w = (util.modifier_weights(5, 3, 40, 12) + 0.3).to(dtype)
+    pc = kind.endswith("PER_CHANNEL")
+    std = WO.weight_std(util.np32(w), pc)
+    np.testing.assert_allclose(std, util.np32(w).astype(np.float64).std(axis=1 if pc else (1, 2), ddof=1,
+                                                                        keepdims=True), rtol=1e-6)
+    np.testing.assert_allclose(std, util.np32(w.float().std(1 if pc else (1, 2), keepdim=True)), rtol=1e-5)
+    # moe_layer_aihwkit_lightning.py:529-541 evaluated by torch
+    bound = 2.0 * w.std(1 if pc else (1, 2), keepdim=True)
+    want = torch.minimum(torch.maximum(w, -bound), bound)
+    got = WO.clip_weights(util.np32(w), kind, 2.0, "bf16" if dtype == torch.bfloat16 else "f32")
+    if dtype == torch.float32:
+        np.testing.assert_allclose(got, util.np32(want), rtol=1e-6)           # std: fp64 here, fp32 in torch
+        assert (got == util.np32(want)).mean() > 0.9
+    else:
+        assert np.array_equal(got, util.np32(want))
+    assert np.array_equal(WO.clip_weights(util.np32(w), "NONE", 2.0), util.np32(w))
+    with pytest.raises(ValueError):
+        WO.clip_weights(util.np32(w), "FIXED_VALUE", 2.0)
+
+
+def test_modifier_normals_are_standard_and_keyed():
+    z = WO.modifier_normals(4, 64, 33, 99)
+    assert z.shape == (4, 64, 33) and abs(z.mean()) < 0.03 and abs(z.std() - 1) < 0.03
+    assert np.array_equal(z, WO.modifier_normals(4, 64, 33, 99)) and not np.array_equal(z, WO.modifier_normals(4, 64, 33, 100))
+    assert not np.array_equal(z[:, :, :32].reshape(256, 32), O.counter_noise(np.arange(256), 32, 0, 99))

@@ -239,3 +239,84 @@ def check_clipped_input_output(ops, device="cpu", dtype=torch.float32, T=100, D=
     a = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
     b = ops.cvmm_bwd_w(p1, dy, E, offsets, perm, tok, ir=ir_dn, ir_by_expert=True, g_scale=gate)
     assert torch.equal(a, b)
+
+
+# ---------------------------------------------------------------------------------- weight modifier / clip
+MODIFIER_KINDS = ("DISCRETIZE", "DISCRETIZE_PER_CHANNEL", "ADD_NORMAL", "ADD_NORMAL_PER_CHANNEL",
+                  "DISCRETIZE_ADD_NORMAL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL")
+
+
+def modifier_weights(seed, E, K, N, dtype=torch.float32, device="cpu"):
+    """Weights with one loud channel and one loud expert, so that per-expert and per-channel maxima differ."""
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(E, K, N, generator=g) * 0.1
+    w[:, :, 0] *= 7.0
+    w[E - 1] *= 3.0
+    return w.to(dtype).to(device)
+
+
+def check_modify_weight(ops, kind, dtype=torch.float32, device="cpu", E=3, K=40, N=24, res=14.0, std_dev=0.07,
+                        seed=0x51EDC0DE12345):
+    """The kernel against the oracle, bit for bit: once with injected normals, once with its own draws."""
+    from oracle import weights_oracle as WO
+    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    w = modifier_weights(7, E, K, N, dtype, device)
+    per_channel = kind in WO.PER_CHANNEL_WMAX
+    wmax = ops.weight_abs_max(w, per_channel)
+    n_states = max(res, 1 / res) if kind.startswith("DISCRETIZE") else 0.0
+    sd = std_dev if "ADD_NORMAL" in kind else 0.0
+    z = torch.randn(E, K, N, generator=torch.Generator().manual_seed(3)).to(dtype)
+    got = ops.modify_weight(w, wmax, n_states, sd, noise=z.float().to(device) if sd > 0 else None)
+    want = WO.modify_weight(np32(w), kind, res, std_dev, np32(z), name)
+    assert got.dtype == dtype and np.array_equal(np32(got), want), kind
+    if sd > 0:
+        got2 = ops.modify_weight(w, wmax, n_states, sd, noise_seed=seed)
+        want2 = WO.modify_weight(np32(w), kind, res, std_dev, WO.modifier_normals(E, K, N, seed), name)
+        # the generator's log2 / sin / cos are hardware approximations: the normals agree to ~1e-6, and in bf16 a
+        # sum that lands within that of a rounding boundary may fall to the other side
+        err = np.abs(np32(got2) - want2)
+        noise_err = 1e-5 * std_dev * float(np32(wmax).max())
+        if dtype == torch.bfloat16:
+            assert err.max() <= 2.0 ** -7 * np.abs(want2).max() and (err > 0).mean() < 0.02, (kind, err.max())
+        else:
+            assert err.max() <= noise_err, (kind, err.max(), noise_err)
+        d = (np32(got2) - WO.modify_weight(np32(w), kind.replace("_ADD_NORMAL", "").replace("ADD_NORMAL", "NONE")
+                                           .replace("NONE_PER_CHANNEL", "NONE"), res, 0.0, None, name))
+        scale = std_dev * np32(wmax).reshape(E, 1, -1)
+        assert abs((d / scale).std() - 1.0) < 0.1 and abs((d / scale).mean()) < 0.1
+        assert not torch.equal(got2, ops.modify_weight(w, wmax, n_states, sd, noise_seed=seed + 1))
+    return got
+
+
+def check_weight_clip(ops, per_channel, dtype=torch.float32, device="cpu", E=3, K=50, N=20, sigma=1.5):
+    from oracle import weights_oracle as WO
+    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    w = (modifier_weights(9, E, K, N) + 0.5).to(dtype).to(device)       # a mean far from zero
+    std = ops.weight_std(w, per_channel)
+    want_std = WO.weight_std(np32(w), per_channel)
+    assert std.shape == want_std.shape
+    np.testing.assert_allclose(np32(std), want_std, rtol=2e-7)
+    before = w.clone()
+    bound = sigma * std.to(dtype)
+    out = ops.clamp_weights_(w, bound)
+    assert out is w
+    kind = "LAYER_GAUSSIAN_PER_CHANNEL" if per_channel else "LAYER_GAUSSIAN"
+    # the clamp itself is exact; against the oracle the bound may sit one ulp away where the two exact sums of
+    # the std round to different fp32 neighbours
+    b = np32(bound).reshape(E, 1, -1)
+    assert np.array_equal(np32(w), np.minimum(np.maximum(np32(before), -b), b))
+    want = WO.clip_weights(np32(before), kind, sigma, name)
+    if dtype == torch.float32:
+        np.testing.assert_allclose(np32(w), want, rtol=3e-7, atol=0)
+    assert (np32(w) == want).mean() > 0.999
+    assert not torch.equal(w, before)
+
+
+def check_weight_abs_max(ops, device="cpu"):
+    """Per-expert and per-channel max |w| over shapes that exercise one lane group per row, several rows per wave,
+    several column blocks and ragged rows."""
+    for E, K, N, dtype in [(3, 70, 20, torch.float32), (2, 300, 256, torch.bfloat16), (2, 37, 520, torch.float32),
+                           (5, 9, 13, torch.bfloat16), (1, 1, 1, torch.float32), (2, 1030, 8, torch.bfloat16)]:
+        w = modifier_weights(E + K, E, K, N, dtype, device)
+        assert torch.equal(ops.weight_abs_max(w, True), w.abs().amax(1).float()), (E, K, N)
+        assert torch.equal(ops.weight_abs_max(w, False), w.abs().amax((1, 2)).float().reshape(E, 1)), (E, K, N)
