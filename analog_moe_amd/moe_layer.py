@@ -316,32 +316,57 @@ def _gaussian_clip_(w: Tensor, sigma: float, per_channel: bool, max_bound: float
     ops.clamp_weights_(w, bound)
 
 
-def load_state_dict_pre_hook(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
-    """Accept checkpoints written by the traceable layout (per-expert ``keys.{i}.input_range``
-    entries, moe_layer_aihwkit_lightning.py:66-105) by folding them into ``input_range [2, E]``."""
+def non_traceable_to_traceable(state_dict, prefix: str = "") -> None:
+    """In place: ``input_range [2, E]`` and its counter become the per-expert entries of the reference's
+    traceable layout -- ``keys.{i}.input_range``, ``.input_range_update_idx``, ``.x_min``, ``.x_max`` and the same
+    under ``values.{i}`` (moe_layer_aihwkit_lightning.py:33-63).  Input ranges of a K-tile split layer
+    ([2, E, n_tiles]) have no counterpart in that layout and are refused."""
+    input_range = state_dict[prefix + "input_range"]
+    update_idx = state_dict[prefix + "input_range_update_idx"]
+    if input_range.dim() != 2:
+        raise MoEConifgError("the traceable layout holds one input range per expert and projection")
+    for i in range(input_range.size(1)):
+        for row, name in enumerate(("keys", "values")):
+            state_dict[prefix + f"{name}.{i}.input_range"] = input_range[row, i].view(1)
+            state_dict[prefix + f"{name}.{i}.input_range_update_idx"] = update_idx.view(1)
+            state_dict[prefix + f"{name}.{i}.x_min"] = torch.zeros(1, device=input_range.device, dtype=input_range.dtype)
+            state_dict[prefix + f"{name}.{i}.x_max"] = torch.zeros(1, device=input_range.device, dtype=input_range.dtype)
+    state_dict.pop(prefix + "input_range")
+    state_dict.pop(prefix + "input_range_update_idx")
+
+
+def traceable_to_non_traceable(state_dict, prefix: str = "") -> None:
+    """In place, the inverse (moe_layer_aihwkit_lightning.py:66-105): per-expert entries, in expert order, are
+    stacked into ``input_range [2, E]``; the counter is taken from the first entry; ``x_min`` / ``x_max`` go."""
     import re
-    if prefix + "input_range" in state_dict:
-        return
-    pat = re.compile(rf"^{re.escape(prefix)}(keys|values)\.(\d+)\.input_range$")
-    found = {}
+    pat = re.compile(rf"^{re.escape(prefix)}(keys|values)\.(\d+)\.(input_range|input_range_update_idx|x_min|x_max)$")
+    found, idx, drop = {}, None, []
     for key in list(state_dict):
         m = pat.match(key)
-        if m:
+        if not m:
+            continue
+        drop.append(key)
+        if m.group(3) == "input_range":
             found[(m.group(1), int(m.group(2)))] = state_dict[key]
+        elif m.group(3) == "input_range_update_idx" and idx is None:
+            idx = state_dict[key]
     if not found:
         return
     n = 1 + max(i for _, i in found)
     state_dict[prefix + "input_range"] = torch.stack([
         torch.cat([found[("keys", i)].reshape(1) for i in range(n)]),
         torch.cat([found[("values", i)].reshape(1) for i in range(n)])])
-    idx_key = next((k for k in state_dict if re.match(
-        rf"^{re.escape(prefix)}(keys|values)\.\d+\.input_range_update_idx$", k)), None)
-    if idx_key is not None:
-        state_dict[prefix + "input_range_update_idx"] = state_dict[idx_key].reshape(())
-    for key in list(state_dict):
-        if re.match(rf"^{re.escape(prefix)}(keys|values)\.\d+\.(input_range|input_range_update_idx|x_min|x_max)$",
-                    key):
-            state_dict.pop(key)
+    if idx is not None:
+        state_dict[prefix + "input_range_update_idx"] = idx.reshape(())
+    for key in drop:
+        state_dict.pop(key)
+
+
+def load_state_dict_pre_hook(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+    """Accept checkpoints written in the traceable layout (moe_layer_aihwkit_lightning.py:108-131; this package
+    has the non-traceable layer only, so that is the one direction a load can need)."""
+    if prefix + "input_range" not in state_dict:
+        traceable_to_non_traceable(state_dict, prefix)
 
 
 class AnalogSigmaMoELayer(SigmaMoELayer):

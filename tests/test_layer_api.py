@@ -60,6 +60,28 @@ def test_loads_traceable_checkpoint_layout():
     assert float(layer.input_range_update_idx) == 5.0
 
 
+def test_state_dict_layout_conversion_round_trip():
+    """moe_layer_aihwkit_lightning.py:33-105, both directions."""
+    from analog_moe_amd.moe_layer import non_traceable_to_traceable, traceable_to_non_traceable
+    layer = AnalogSigmaMoELayer(_rpu(), d_model=8, n_experts=3, expert_size=4, k=1, analog_router=False)
+    layer.input_range.data = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    layer.input_range_update_idx.data.fill_(7.0)
+    sd = {"blk." + k: v.clone() for k, v in layer.state_dict().items()}
+    non_traceable_to_traceable(sd, "blk.")
+    assert "blk.input_range" not in sd and "blk.input_range_update_idx" not in sd
+    assert sd["blk.keys.1.input_range"].tolist() == [2.0] and sd["blk.values.2.input_range"].tolist() == [6.0]
+    assert sd["blk.values.0.input_range_update_idx"].tolist() == [7.0] and sd["blk.keys.2.x_max"].tolist() == [0.0]
+    assert len([k for k in sd if ".input_range" in k or ".x_m" in k]) == 3 * 2 * 4
+    traceable_to_non_traceable(sd, "blk.")
+    want = {"blk." + k: v for k, v in layer.state_dict().items()}
+    assert sd.keys() == want.keys() and all(torch.equal(sd[k], want[k]) for k in want)
+    split = _rpu()
+    split.mapping.max_input_size = 4
+    tiled = AnalogSigmaMoELayer(split, d_model=8, n_experts=2, expert_size=4, k=1, analog_router=False)
+    with pytest.raises(MoEConifgError):
+        non_traceable_to_traceable(dict(tiled.state_dict()))
+
+
 def test_tile_split_gives_per_tile_ranges():
     r = _rpu()
     r.mapping.max_input_size = 512
