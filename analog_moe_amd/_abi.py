@@ -83,6 +83,9 @@ PROTOTYPES = {
     "amoe_weight_std_workspace": (SZ, [I32, I32, I32, I32]),
     "amoe_weight_std": (C.c_int, [I32, P, I32, I32, I32, I32, P, P, SZ, P]),
     "amoe_clamp_weights": (C.c_int, [I32, P, I32, I32, I32, P, I32, P]),
+    "amoe_select_workspace": (SZ, [I64, I32]),
+    "amoe_select_fwd": (C.c_int, [I32, P, I64, I32, I32, P, P, P, P, P, SZ, P]),
+    "amoe_select_bwd": (C.c_int, [I32, P, I64, I32, I32, P, P, P, P, P, P]),
 }
 
 

@@ -5,6 +5,7 @@
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
 #include "weight_kernels.h"
+#include "select_kernels.h"
 #include "prepare_sel.h"
 
 using namespace amoe;
@@ -687,6 +688,100 @@ int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N, 
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<uint16_t*>(w), bound, rows,
                        (int)K, (int)N, (int)cols, vec, cvec);
   }
+  return launch_rc();
+}
+
+static long long select_blocks(long long T) { return (T + 4 * kSelRowsPerWave - 1) / (4 * kSelRowsPerWave); }
+
+size_t amoe_select_workspace(int64_t T, int32_t E) {
+  if (T < 1 || E < 1) return 0;
+  const long long blocks = select_blocks(T);
+  return (size_t)(blocks + (blocks + kSelSumChunk - 1) / kSelSumChunk) * E * sizeof(float);
+}
+
+int amoe_select_fwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k, void* sel_val, int64_t* sel_idx,
+                    float* reg, float* reg_c, void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (T < 0 || E < 1 || k < 1 || k > E) return AMOE_EINVAL;
+  if (E > 64 * kSelPerLane) return AMOE_EUNSUPPORTED;
+  if (T == 0) return AMOE_OK;
+  if (!logits || !sel_val || !sel_idx) return AMOE_ENULL;
+  if ((reg != nullptr) != (reg_c != nullptr)) return AMOE_EINVAL;
+  if (!aligned(logits, esize(dtype)) || !aligned(sel_val, esize(dtype)) || !aligned(sel_idx, 8) || !aligned(reg, 4) ||
+      !aligned(reg_c, 4) || !aligned(workspace, 4))
+    return AMOE_EALIGN;
+  const long long blocks = select_blocks(T);
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  float* partial = nullptr;
+  if (reg != nullptr) {
+    if (!workspace) return AMOE_ENULL;
+    if (workspace_bytes < amoe_select_workspace(T, E)) return AMOE_EWORKSPACE;
+    partial = static_cast<float*>(workspace);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define AMOE_SELECT_FWD(PER)                                                                                           \
+  do {                                                                                                                 \
+    if (dtype == AMOE_F32) {                                                                                           \
+      auto kf = &select_fwd_kernel<float, PER>;                                                                        \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(logits),         \
+                         (long long)T, (int)E, (int)k, static_cast<float*>(sel_val), sel_idx, partial);                \
+    } else {                                                                                                           \
+      auto kf = &select_fwd_kernel<uint16_t, PER>;                                                                     \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(logits),      \
+                         (long long)T, (int)E, (int)k, static_cast<uint16_t*>(sel_val), sel_idx, partial);             \
+    }                                                                                                                  \
+  } while (0)
+  if (E <= 64) AMOE_SELECT_FWD(1);
+  else if (E <= 128) AMOE_SELECT_FWD(2);
+  else if (E <= 256) AMOE_SELECT_FWD(4);
+  else AMOE_SELECT_FWD(8);
+#undef AMOE_SELECT_FWD
+  if (int rc = launch_rc()) return rc;
+  if (reg != nullptr) {
+    const int groups = (int)((blocks + kSelSumChunk - 1) / kSelSumChunk);
+    float* level2 = partial + blocks * E;
+    hipLaunchKernelGGL(select_usage_sum_kernel, dim3(groups), dim3(kThreads), 0, st, partial, (int)blocks, (int)E, level2);
+    if (int rc = launch_rc()) return rc;
+    hipLaunchKernelGGL(select_reg_kernel, dim3(1), dim3(kThreads), 0, st, level2, groups, (int)E, (long long)T, reg,
+                       reg_c);
+    return launch_rc();
+  }
+  return AMOE_OK;
+}
+
+int amoe_select_bwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k, const int64_t* sel_idx,
+                    const void* grad_val, const float* reg_c, const float* grad_reg, void* grad_logits, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (T < 0 || E < 1 || k < 1 || k > E) return AMOE_EINVAL;
+  if (E > 64 * kSelPerLane) return AMOE_EUNSUPPORTED;
+  if (T == 0) return AMOE_OK;
+  if (!logits || !grad_logits || (grad_val && !sel_idx)) return AMOE_ENULL;
+  if ((reg_c != nullptr) != (grad_reg != nullptr)) return AMOE_EINVAL;
+  if (!aligned(logits, esize(dtype)) || !aligned(grad_logits, esize(dtype)) || !aligned(grad_val, esize(dtype)) ||
+      !aligned(sel_idx, 8) || !aligned(reg_c, 4) || !aligned(grad_reg, 4))
+    return AMOE_EALIGN;
+  const long long blocks = (T + 3) / 4;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define AMOE_SELECT_BWD(PER)                                                                                           \
+  do {                                                                                                                 \
+    if (dtype == AMOE_F32) {                                                                                           \
+      auto kf = &select_bwd_kernel<float, PER>;                                                                        \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(logits),         \
+                         (long long)T, (int)E, (int)k, sel_idx, static_cast<const float*>(grad_val), reg_c, grad_reg,  \
+                         static_cast<float*>(grad_logits));                                                            \
+    } else {                                                                                                           \
+      auto kf = &select_bwd_kernel<uint16_t, PER>;                                                                     \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(logits),      \
+                         (long long)T, (int)E, (int)k, sel_idx, static_cast<const uint16_t*>(grad_val), reg_c,         \
+                         grad_reg, static_cast<uint16_t*>(grad_logits));                                               \
+    }                                                                                                                  \
+  } while (0)
+  if (E <= 64) AMOE_SELECT_BWD(1);
+  else if (E <= 128) AMOE_SELECT_BWD(2);
+  else if (E <= 256) AMOE_SELECT_BWD(4);
+  else AMOE_SELECT_BWD(8);
+#undef AMOE_SELECT_BWD
   return launch_rc();
 }
 

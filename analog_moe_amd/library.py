@@ -11,6 +11,7 @@ so every group of calls the Python layer makes is one opaque operator with a fak
   amoe::expert_std          per-expert std                    (cvmm.py:400-443)
   amoe::weight_abs_max      max |W| per expert / per channel  (moe_layer_aihwkit_lightning.py:476-489)
   amoe::modify_weight       weight modifier of a forward      (moe_layer_aihwkit_lightning.py:313-382)
+  amoe::select / select_bwd sigmoid + top-k + usage regulariser of the router's logits
   amoe::cvmm_forward        everything CVMM.forward launches  (cvmm.py:701-769)
   amoe::cvmm_backward       everything CVMM.backward launches (cvmm.py:772-897)
   amoe::ffn_fwd / ffn_bwd   the fused expert feed-forward, with its autograd formula registered
@@ -145,6 +146,55 @@ def _modify_autograd(ctx, grad):
 
 
 modify_weight.register_autograd(_modify_autograd)
+
+
+# --------------------------------------------------------------------------- router epilogue
+@torch.library.custom_op("amoe::select", mutates_args=(),
+                         schema="(Tensor logits, int k, bool want_reg) -> (Tensor, Tensor, Tensor, Tensor)")
+def select(logits, k, want_reg):
+    """(sel_val [T, k], sel_idx [T, k] int64, reg, reg_c): sigmoid gate values and ids of the top-k experts per
+    row of logits [T, E], and the usage regulariser with its derivative table (empty without want_reg)."""
+    return ops.select_fwd(logits, k, want_reg)
+
+
+@select.register_fake
+def _(logits, k, want_reg):
+    T, E = logits.shape
+    f32 = dict(dtype=torch.float32, device=logits.device)
+    return (logits.new_empty((T, k)), torch.empty((T, k), dtype=torch.int64, device=logits.device),
+            torch.empty((), **f32) if want_reg else torch.empty(_EMPTY_SHAPE, **f32),
+            torch.empty(E if want_reg else 0, **f32))
+
+
+@torch.library.custom_op("amoe::select_bwd", mutates_args=(),
+                         schema="(Tensor logits, Tensor sel_idx, Tensor? grad_val, Tensor? reg_c, Tensor? grad_reg) -> Tensor")
+def select_bwd(logits, sel_idx, grad_val, reg_c, grad_reg):
+    return ops.select_bwd(logits, sel_idx, grad_val, reg_c, grad_reg)
+
+
+@select_bwd.register_fake
+def _(logits, sel_idx, grad_val, reg_c, grad_reg):
+    return torch.empty_like(logits)
+
+
+def _select_setup_context(ctx, inputs, output):
+    logits, k, want_reg = inputs
+    _, sel_idx, _, reg_c = output
+    ctx.save_for_backward(logits, sel_idx, reg_c)
+    ctx.want_reg = want_reg
+    ctx.set_materialize_grads(False)
+
+
+def _select_autograd(ctx, grad_val, _grad_idx, grad_reg, _grad_c):
+    logits, sel_idx, reg_c = ctx.saved_tensors
+    if grad_val is None and (grad_reg is None or not ctx.want_reg):
+        return None, None, None
+    with_reg = ctx.want_reg and grad_reg is not None
+    return (torch.ops.amoe.select_bwd(logits, sel_idx, grad_val, reg_c if with_reg else None,
+                                      grad_reg if with_reg else None), None, None)
+
+
+select.register_autograd(_select_autograd, setup_context=_select_setup_context)
 
 
 # --------------------------------------------------------------------------- CVMM forward / backward

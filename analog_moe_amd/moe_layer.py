@@ -115,6 +115,12 @@ class SigmaMoELayer(nn.Module):
     def select(self, x: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
         """Gate values and expert ids [..., k] of the top-k experts, and the regularisation loss."""
         logits = self.expert_sel(x)
+        if self._fused_select(logits):
+            # sigmoid, top-k and the regulariser in one pass over the logits (and one for their gradient)
+            val, idx, reg, _ = torch.ops.amoe.select(logits.reshape(-1, self.n_experts), self.n_heads, self.training)
+            lead = logits.shape[:-1]
+            return (val.view(*lead, self.n_heads), idx.view(*lead, self.n_heads),
+                    reg if self.training else x.new_zeros(()))
         reg_loss = x.new_zeros(())
         if self.training and logits.numel() > 0:
             logp = F.log_softmax(logits.float(), dim=-1).flatten(end_dim=-2)
@@ -128,6 +134,13 @@ class SigmaMoELayer(nn.Module):
         if self.activation_after_topk:
             sel_val = self._sel_activation(sel_val)
         return sel_val, sel_idx, reg_loss
+
+    def _fused_select(self, logits: Tensor) -> bool:
+        """The plain router (sigmoid before top-k, no expert dropout) on the GPU takes the fused kernels."""
+        return ((logits.is_cuda or logits.is_meta) and self.selection_mode == "sigmoid"
+                and not self.activation_after_topk and not (self.training and self.expert_dropout > 0)
+                and self.n_heads <= self.n_experts <= ops.SELECT_MAX_EXPERTS and logits.numel() > 0
+                and logits.dtype in (torch.float32, torch.bfloat16))
 
     def _sel_activation(self, t: Tensor) -> Tensor:
         return torch.sigmoid(t) if self.selection_mode == "sigmoid" else F.softmax(t, dim=-1)

@@ -273,3 +273,42 @@ def clamp_weights_(w: torch.Tensor, bound: torch.Tensor) -> torch.Tensor:
         raise ValueError("bound must hold one value per expert or per expert and channel")
     raw.clamp_weights(get_lib(), _stream(w), w.detach(), _f32c(bound), cols)
     return w
+
+
+# ------------------------------------------------------------------------------ router epilogue
+SELECT_MAX_EXPERTS = 512
+
+
+def select_fwd(logits: torch.Tensor, k: int, want_reg: bool):
+    """Gate values [T, k] and expert ids [T, k] (int64) of the k largest sigmoid(logits) per row; with want_reg also
+    the usage regulariser (fp32 scalar) and its derivative table [E] for ``select_bwd`` (else two empty tensors)."""
+    _need_gpu(logits)
+    lib = get_lib()
+    lg = logits.detach().contiguous()
+    T, E = lg.shape
+    sel_val = torch.empty((T, k), dtype=lg.dtype, device=lg.device)
+    sel_idx = torch.empty((T, k), dtype=torch.int64, device=lg.device)
+    reg = reg_c = ws = None
+    if want_reg:
+        reg = torch.empty((), dtype=torch.float32, device=lg.device)
+        reg_c = torch.empty(E, dtype=torch.float32, device=lg.device)
+        ws = torch.empty(max(lib.amoe_select_workspace(T, E) // 4, 1), dtype=torch.float32, device=lg.device)
+    raw.select_fwd(lib, _stream(lg), lg, k, sel_val, sel_idx, reg, reg_c, ws)
+    if not want_reg:
+        reg = torch.empty(0, dtype=torch.float32, device=lg.device)
+        reg_c = torch.empty(0, dtype=torch.float32, device=lg.device)
+    return sel_val, sel_idx, reg, reg_c
+
+
+def select_bwd(logits: torch.Tensor, sel_idx: torch.Tensor, grad_val: Optional[torch.Tensor],
+               reg_c: Optional[torch.Tensor], grad_reg: Optional[torch.Tensor]) -> torch.Tensor:
+    _need_gpu(logits, sel_idx, grad_val, reg_c, grad_reg)
+    lg = logits.detach().contiguous()
+    out = torch.empty_like(lg)
+    if lg.numel() == 0:
+        return out
+    gv = None if grad_val is None else grad_val.detach().to(lg.dtype).contiguous()
+    gr = None if grad_reg is None else grad_reg.detach().to(torch.float32).reshape(1).contiguous()
+    raw.select_bwd(get_lib(), _stream(lg), lg, sel_idx.shape[-1], sel_idx.contiguous(), gv,
+                   None if gr is None else reg_c, gr, out)
+    return out

@@ -268,3 +268,24 @@ def clamp_weights(lib, stream, w, bound, cols: int):
         raise ValueError("bound must be [E] or [E, N]")
     check(lib, lib.amoe_clamp_weights(dtype_code(w), _p(w), E, K, N, _p(_f32(bound, "bound")), cols, stream),
           "amoe_clamp_weights")
+
+
+def select_fwd(lib, stream, logits, k: int, sel_val, sel_idx, reg, reg_c, workspace):
+    T, E = logits.shape
+    if not logits.is_contiguous() or sel_idx.dtype != torch.int64 or sel_val.dtype != logits.dtype:
+        raise ValueError("logits must be contiguous, sel_val of its dtype, sel_idx int64")
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    check(lib, lib.amoe_select_fwd(dtype_code(logits), _p(logits), T, E, k, _p(sel_val), _p(sel_idx),
+                                   _p(_f32(reg, "reg")), _p(_f32(reg_c, "reg_c")), _p(workspace), nbytes, stream),
+          "amoe_select_fwd")
+
+
+def select_bwd(lib, stream, logits, k: int, sel_idx, grad_val, reg_c, grad_reg, grad_logits):
+    T, E = logits.shape
+    if not logits.is_contiguous() or not grad_logits.is_contiguous():
+        raise ValueError("logits and grad_logits must be contiguous")
+    if grad_val is not None and (grad_val.dtype != logits.dtype or not grad_val.is_contiguous()):
+        raise ValueError("grad_val must be contiguous and of the logits' dtype")
+    check(lib, lib.amoe_select_bwd(dtype_code(logits), _p(logits), T, E, k, _p(sel_idx), _p(grad_val),
+                                   _p(_f32(reg_c, "reg_c")), _p(_f32(grad_reg, "grad_reg")), _p(grad_logits), stream),
+          "amoe_select_bwd")

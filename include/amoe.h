@@ -273,6 +273,26 @@ int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t 
 int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N,
                        const float* bound, int32_t cols, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Router epilogue: gate values and top-k experts of every token from the router's logits
+ * [T, E], and the regulariser of the mean expert usage.  The reference's layer inherits this
+ * step from sigma_moe.SigmaMoELayer (absent from the checkout); its per-token form is
+ * tests/test_moe_layer_aihwkit_lightning.py:82-90: sel = sigmoid(expert_sel(x));
+ * sel_val, sel_idx = sel.topk(k, dim=-1, sorted=False).
+ *   sel_val [T, k] (dtype), sel_idx [T, k] int64: descending gate value, ties to the lower id
+ *   reg (optional, fp32 scalar): sum_e pbar_e log pbar_e, pbar = mean_t softmax(logits[t])
+ *   reg_c (with reg, fp32 [E]): 1 + log pbar_e, which amoe_select_bwd reads
+ * E <= 512.  workspace: amoe_select_workspace bytes when reg is asked for. */
+size_t amoe_select_workspace(int64_t T, int32_t E);
+int amoe_select_fwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k,
+                    void* sel_val, int64_t* sel_idx, float* reg, float* reg_c,
+                    void* workspace, size_t workspace_bytes, void* stream);
+/* grad_logits [T, E] from grad_val [T, k] (optional) through the sigmoid of the chosen experts and
+ * from *grad_reg (device fp32 scalar, optional, with reg_c) through the regulariser. */
+int amoe_select_bwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k,
+                    const int64_t* sel_idx, const void* grad_val, const float* reg_c,
+                    const float* grad_reg, void* grad_logits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -156,6 +156,15 @@ def test_weight_std_and_clamp_match_oracle(emu_ops, per_channel, dtype):
         util.check_weight_clip(emu_ops, per_channel, dtype, E=2, K=300, N=200)   # several slices per expert
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_epilogue_matches_oracle(emu_ops, dtype):
+    util.check_select(emu_ops, dtype)
+    util.check_select(emu_ops, dtype, T=33, E=130, k=8, seed=1)           # three experts per lane, a ragged last wave
+    util.check_select(emu_ops, dtype, T=5, E=2, k=2, seed=2)
+    util.check_select(emu_ops, dtype, T=9, E=100, k=4, seed=3)            # two experts per lane
+    util.check_select(emu_ops, dtype, T=9, E=300, k=5, seed=4)            # eight (five used)
+
+
 def test_transposed_weight_view(emu_ops):
     """cvmm.py:839 hands the forward launcher `keys.transpose(1, 2)`: k-contiguous weights."""
     pr = util.make_problem(13, T=30, D=72, E=3, F=40, k=2)

@@ -670,3 +670,45 @@ def test_aihwkit_flavour_modifier_and_clip_on_the_gpu():
     layer.reset_parameters()
     layer.clip_weights(cfgmod.WeightClipParameter(type=cfgmod.WeightClipType.LAYER_GAUSSIAN, sigma=5.0, fixed_value=0.02))
     assert layer.keys.data.abs().max().item() <= 0.02 + 1e-7
+
+
+# ---------------------------------------------------------------------------------- router epilogue kernels
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_epilogue_kernels_match_oracle(dtype):
+    from analog_moe_amd import ops
+    util.check_select(ops, dtype, device="cuda")
+    util.check_select(ops, dtype, device="cuda", T=33, E=130, k=8, seed=1)
+    util.check_select(ops, dtype, device="cuda", T=4096, E=64, k=8, seed=2)
+    util.check_select(ops, dtype, device="cuda", T=5, E=2, k=2, seed=3)
+    util.check_select(ops, dtype, device="cuda", T=100, E=100, k=4, seed=4)
+    util.check_select(ops, dtype, device="cuda", T=100, E=300, k=5, seed=5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_router_epilogue_equals_the_tensor_expression(dtype):
+    """The layer's select() through amoe::select against the same layer with the kernels switched off (sigmoid,
+    topk, log_softmax / logsumexp in torch): gate values, chosen experts, regulariser and the router's gradient."""
+    from analog_moe_amd import config as cfgmod
+    res = []
+    for fused in (True, False):
+        layer = _layer(cfgmod, dict(analog_router=False), dtype=dtype)
+        if not fused:
+            layer._fused_select = lambda logits: False
+        layer.train()
+        torch.manual_seed(3)
+        x = torch.randn(6, 50, 128, device="cuda", dtype=dtype)
+        val, idx, reg = layer.select(x)
+        w = torch.linspace(-1, 1, val.numel(), device="cuda").view_as(val).to(dtype)
+        ((val * w).sum().float() + 0.5 * reg.float()).backward()
+        order = idx.argsort(-1)
+        res.append((val.gather(-1, order).float(), idx.gather(-1, order), reg.float(),
+                    layer.expert_sel.weight.grad.float().clone()))
+    (v1, i1, r1, g1), (v0, i0, r0, g0) = res
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    same = (i1 == i0).all(-1)
+    assert same.float().mean() > 0.99                      # rows with tied gate values may choose another expert
+    assert torch.allclose(v1[same], v0[same], rtol=tol, atol=tol)
+    assert torch.allclose(r1, r0, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(g1, g0, rtol=10 * tol, atol=10 * tol * g0.abs().max().item())
+    layer.eval()
+    assert float(layer.select(x)[2]) == 0.0

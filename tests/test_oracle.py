@@ -463,3 +463,47 @@ def test_modifier_normals_are_standard_and_keyed():
     assert z.shape == (4, 64, 33) and abs(z.mean()) < 0.03 and abs(z.std() - 1) < 0.03
     assert np.array_equal(z, WO.modifier_normals(4, 64, 33, 99)) and not np.array_equal(z, WO.modifier_normals(4, 64, 33, 100))
     assert not np.array_equal(z[:, :, :32].reshape(256, 32), O.counter_noise(np.arange(256), 32, 0, 99))
+
+
+# ---------------------------------------------------------------------------------- router epilogue
+from oracle import select_oracle as SO   # noqa: E402
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_select_oracle_matches_torch_sigmoid_topk(dtype):
+    """tests/test_moe_layer_aihwkit_lightning.py:85-87 evaluated by torch on the CPU."""
+    torch.manual_seed(0)
+    logits = (torch.randn(200, 32) * 2).to(dtype)
+    sel = torch.sigmoid(logits)
+    want_val, want_idx = sel.topk(4, dim=-1, sorted=False)
+    val, idx = SO.select(util.np32(logits), 4, "bf16" if dtype == torch.bfloat16 else "f32")
+    # sorted=False leaves the order open and ties may go to another id: compare the values as sets per row, and
+    # the values behind the oracle's ids
+    ref = np.sort(util.np32(want_val), axis=-1)[:, ::-1]
+    if dtype == torch.bfloat16:
+        assert np.array_equal(val, ref)
+        assert np.array_equal(np.take_along_axis(util.np32(sel), idx, -1), val)
+    else:
+        np.testing.assert_allclose(val, ref, rtol=2e-7)
+    assert (np.diff(val, axis=-1) <= 0).all() and all(len(set(r)) == 4 for r in idx.tolist())
+    tie = SO.select(np.zeros((1, 6), np.float32), 3)[1]
+    assert tie.tolist() == [[0, 1, 2]]
+
+
+def test_regulariser_and_select_bwd_match_torch_autograd():
+    torch.manual_seed(1)
+    logits = (torch.randn(50, 12) * 2).requires_grad_()
+    logp = torch.log_softmax(logits, dim=-1)
+    mean_logp = torch.logsumexp(logp, dim=0) - np.log(50)
+    reg = (mean_logp.exp() * mean_logp).sum()
+    val, idx = torch.sigmoid(logits).topk(3, dim=-1)
+    gv = torch.randn(50, 3)
+    ((val * gv).sum() + 0.7 * reg).backward()
+    got_reg, c = SO.usage_regulariser(logits.detach().numpy())
+    assert abs(float(got_reg) - float(reg)) < 1e-6
+    uniform_reg, _ = SO.usage_regulariser(np.zeros((7, 8), np.float32))
+    assert abs(float(uniform_reg) + np.log(8)) < 1e-6                       # uniform usage: minus log E
+    got = SO.select_bwd(logits.detach().numpy(), idx.numpy(), gv.numpy(), 0.7)
+    np.testing.assert_allclose(got, logits.grad.numpy(), rtol=1e-4, atol=1e-7)
+    only_reg = SO.select_bwd(logits.detach().numpy(), idx.numpy(), None, 1.0)
+    np.testing.assert_allclose(only_reg.sum(axis=-1), 0.0, atol=1e-7)       # softmax gradients sum to zero per row

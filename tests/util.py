@@ -320,3 +320,44 @@ def check_weight_abs_max(ops, device="cpu"):
         w = modifier_weights(E + K, E, K, N, dtype, device)
         assert torch.equal(ops.weight_abs_max(w, True), w.abs().amax(1).float()), (E, K, N)
         assert torch.equal(ops.weight_abs_max(w, False), w.abs().amax((1, 2)).float().reshape(E, 1)), (E, K, N)
+
+
+# ---------------------------------------------------------------------------------- router epilogue
+def check_select(ops, dtype=torch.float32, device="cpu", T=70, E=24, k=3, seed=0):
+    """select_fwd / select_bwd against the oracle: gate values bit for bit (the chosen ids carry exactly those
+    values; where gate values tie, the kernel takes the lower id like the oracle), regulariser and gradients to
+    fp32 / bf16 accuracy."""
+    from oracle import select_oracle as SO
+    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    g = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(T, E, generator=g) * 2.0).to(dtype)
+    logits[0, :] = logits[0, 0]                                     # a row of ties
+    dev = logits.to(device)
+    val, idx, reg, reg_c = ops.select_fwd(dev, k, True)
+    want_val, want_idx = SO.select(np32(logits), k, name)
+    # expf differs in the last fp32 bit between the device library, the host library and numpy: fp32 gate values
+    # agree to an ulp (and the order of two experts whose values differ by less may swap), bf16 ones exactly
+    if dtype == torch.bfloat16:
+        assert np.array_equal(np32(val), want_val)
+        assert np.array_equal(idx.cpu().numpy(), want_idx)
+    else:
+        np.testing.assert_allclose(np32(val), want_val, rtol=3e-7)
+        assert (idx.cpu().numpy() == want_idx).mean() > 0.999
+    sig = 1.0 / (1.0 + np.exp(-np32(logits).astype(np.float64)))
+    np.testing.assert_allclose(np.take_along_axis(sig, idx.cpu().numpy(), -1), np32(val),
+                               rtol=1e-2 if dtype == torch.bfloat16 else 1e-6)
+    assert all(len(set(r)) == k for r in idx.cpu().numpy().tolist())
+    want_reg, want_c = SO.usage_regulariser(np32(logits))
+    np.testing.assert_allclose(float(reg), want_reg, rtol=1e-5)
+    np.testing.assert_allclose(np32(reg_c), want_c, rtol=1e-5, atol=1e-6)
+    v2, i2, r2, c2 = ops.select_fwd(dev, k, False)
+    assert torch.equal(v2, val) and torch.equal(i2, idx) and r2.numel() == 0 and c2.numel() == 0
+    gv = torch.randn(T, k, generator=g).to(dtype)
+    greg = torch.tensor(0.7)
+    tol = dict(rtol=2e-2, atol=2e-3) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-6)
+    for use_val, use_reg in ((True, True), (True, False), (False, True)):
+        got = ops.select_bwd(dev, idx, gv.to(device) if use_val else None, reg_c if use_reg else None,
+                             greg.to(device) if use_reg else None)
+        want = SO.select_bwd(np32(logits), idx.cpu().numpy(), np32(gv) if use_val else None,
+                             0.7 if use_reg else None, name)
+        np.testing.assert_allclose(np32(got), want, **tol)
