@@ -222,3 +222,31 @@ def test_full_size_properties(ops, name, T, D, E, F, k, routing):
     want_g = torch.einsum("rn,rkn->rk", dy[tok[pos].long()].double(), values[e_of].double())
     got_g = full[perm[pos].long()].double()
     assert float((got_g - want_g).abs().max() / want_g.abs().max()) < 1e-2
+
+
+@pytest.mark.parametrize("name", ["config1_dac", "config1_dac_adc_split"])
+def test_golden_fixture_parity(ops, name):
+    """The HIP path on the committed inputs against the committed expected outputs (tests/golden/*.npz)."""
+    import os
+    from tests.golden import make_golden as G
+    fx = np.load(os.path.join(os.path.dirname(G.__file__), name + ".npz"))
+    _, _, lk, _ = G.problem(name)
+    pr = {n[3:]: torch.from_numpy(fx[n]) for n in fx.files if n.startswith("in_") and n != "in_ir"}
+    ir = torch.from_numpy(fx["in_ir"])
+    print("fixture", name, flush=True)
+    if lk.get("out_bound", -1) > 0:
+        lk = dict(lk)          # the layer ops take max |W| themselves
+    got = util.layer_ops_fwd_bwd(ops, _to(pr), ir.cuda(), **lk)
+    torch.cuda.synchronize()
+    want = O.LayerOracle(y=fx["out_y"], scores=fx["out_scores"], z=fx["out_z"],
+                         sel=O.SelOracle(*(fx["out_" + n] for n in ("sel_sorted", "perm", "in_index", "offsets"))),
+                         grad_x=fx["out_grad_x"], grad_keys=fx["out_grad_keys"], grad_values=fx["out_grad_values"],
+                         grad_gate=fx["out_grad_gate"], grad_ir=fx["out_grad_ir"])
+    adc = util.adc_steps(pr, ir, lk)
+    if adc is None:
+        print(util.compare_layer(got, want, TOL["f32"]))
+        return
+    # with the output quantiser on, a last-bit difference in a sum moves a value by one ADC step, and what follows
+    # inherits it: the quantised stages are compared with the step allowance, what follows with a wider tolerance
+    errs = util.compare_layer(got, want, 1e-4, adc_step=adc)
+    print(errs)
