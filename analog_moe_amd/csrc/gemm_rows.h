@@ -784,7 +784,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           }
 #pragma unroll
           for (int i = 0; i < NROW; i++)
-            if (orow[i] >= 0) *reinterpret_cast<Raw*>(DST + (int64_t)orow[i] * ldd + c0 + (tid % OCPR) * CH) = seg[i];
+            if (orow[i] >= 0) store_streaming(DST + (int64_t)orow[i] * ldd + c0 + (tid % OCPR) * CH, seg[i]);
         }
         if (xf_stage && p.xc_out != nullptr) {     // the parked input tile, clipped and scaled in place
           const T* __restrict__ sXF = sStage + (sOut == sStage ? STAGE : 0);
@@ -799,7 +799,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
           for (int i = 0; i < NROW; i++)
             if (xrow[i] >= 0)
-              *reinterpret_cast<Raw*>(static_cast<T*>(p.xc_out) + (int64_t)xrow[i] * p.ldxc + c0 + (tid % OCPR) * CH) = seg[i];
+              store_streaming(static_cast<T*>(p.xc_out) + (int64_t)xrow[i] * p.ldxc + c0 + (tid % OCPR) * CH, seg[i]);
         }
         __syncthreads();
       }

@@ -40,8 +40,8 @@ CONFIGS = {
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
 # the counter runs summarised under profiles/; None where not measured
-TRAFFIC = {"c3": {"fwd_up": 530069119, "fwd_down": 473917796, "wgrad_down": 370373459, "wgrad_up": 370391792,
-                  "xgrad_down": 460076506, "xgrad_up": 697656849}}
+TRAFFIC = {"c3": {"fwd_up": 519587214, "fwd_down": 445629650, "wgrad_down": 370370826, "wgrad_up": 370378281,
+                  "xgrad_down": 462804511, "xgrad_up": 640523555}}
 
 
 def cpu_baseline(cfg, pr, budget_tokens):
