@@ -98,6 +98,15 @@ __device__ __forceinline__ Raw raw_load(const T* p, int n_valid, bool vec) {
   return r;
 }
 
+// raw_load for operands that are read exactly once by the whole launch (the k-head tensors of the row-wise
+// companions): a complete, aligned chunk is fetched with the non-temporal hint, so that it does not push the
+// operand tiles of a GEMM launch running beside it out of the L2.
+template <typename T>
+__device__ __forceinline__ Raw raw_load_streaming(const T* p, int n_valid, bool vec) {
+  if (vec && n_valid >= Elem<T>::kChunk) return __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p));
+  return raw_load<T>(p, n_valid, vec);
+}
+
 template <typename T>
 __device__ __forceinline__ void raw_unpack(const Raw& r, float (&v)[Elem<T>::kChunk]) {
   if constexpr (sizeof(T) == 4) {

@@ -456,7 +456,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
           for (int i = 0; i < 8; i++) {
             const int rl = tid / 16 + 16 * i;
-            const Raw v = *reinterpret_cast<const Raw*>(XF + (int64_t)sXrow[rl] * p.ldxf + c0 + (tid % 16) * CH);
+            // (when the clipped input is written back, every row of x belongs to one sorted position and its
+            // segment is read by this item only; token rows shared by k positions are better kept in the L2)
+            const Raw* src = reinterpret_cast<const Raw*>(XF + (int64_t)sXrow[rl] * p.ldxf + c0 + (tid % 16) * CH);
+            const Raw v = p.xc_out != nullptr ? __builtin_nontemporal_load(src) : *src;
             if (i < 4) ra0[i] = v; else rb0[i - 4] = v;
           }
         }

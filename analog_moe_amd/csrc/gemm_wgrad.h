@@ -329,8 +329,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
 #pragma unroll
     for (int i = 0; i < kTileRows / ORPP; i++) {
       const int rl = tid / OCPR + ORPP * i;
-      *reinterpret_cast<Raw*>(GW + (int64_t)(kc0 + rl) * p.N + n0 + (tid % OCPR) * CH) =
-          *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+      store_streaming(GW + (int64_t)(kc0 + rl) * p.N + n0 + (tid % OCPR) * CH,
+                      *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]));
     }
     return;
   }

@@ -24,14 +24,14 @@ __global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restri
   for (int q = 0; q < CH; q++) acc[q] = 0.f;
   for (int j = 0; j < k; j++) {
     float v[CH];
-    raw_unpack<T>(raw_load<T>(z + (t * k + j) * (long long)D + d, nv, vec != 0), v);
+    raw_unpack<T>(raw_load_streaming<T>(z + (t * k + j) * (long long)D + d, nv, vec != 0), v);
     const float gt = gate ? Elem<T>::load(gate + t * k + j) : 1.f;
 #pragma unroll
     for (int q = 0; q < CH; q++) acc[q] += gt * v[q];
   }
   T* out = y + t * (long long)D + d;
   if (vec && nv == CH) {
-    *reinterpret_cast<Raw*>(out) = raw_pack<T>(acc);
+    store_streaming(out, raw_pack<T>(acc));
   } else {
     for (int q = 0; q < nv; q++) out[q] = Elem<T>::cvt(acc[q]);
   }
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict
       Raw ra[JB];
 #pragma unroll
       for (int jj = 0; jj < JB; jj++)
-        ra[jj] = j0 + jj < k ? raw_load<T>(z + (t * k + j0 + jj) * (long long)D + d, nv, vec != 0) : raw_zero();
+        ra[jj] = j0 + jj < k ? raw_load_streaming<T>(z + (t * k + j0 + jj) * (long long)D + d, nv, vec != 0) : raw_zero();
       float b[CH];
       raw_unpack<T>(raw_load<T>(dr + d, nv, vec != 0), b);
 #pragma unroll

@@ -40,8 +40,8 @@ CONFIGS = {
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
 # the counter runs summarised under profiles/; None where not measured
-TRAFFIC = {"c3": {"fwd_up": 519587214, "fwd_down": 445629650, "wgrad_down": 370370826, "wgrad_up": 370378281,
-                  "xgrad_down": 462804511, "xgrad_up": 640523555}}
+TRAFFIC = {"c3": {"fwd_up": 518229781, "fwd_down": 440371620, "wgrad_down": 370374685, "wgrad_up": 370383451,
+                  "xgrad_down": 478628453, "xgrad_up": 640301186}}
 
 
 def cpu_baseline(cfg, pr, budget_tokens):
