@@ -303,5 +303,27 @@ def test_library_rejects_bad_arguments_on_the_host():
     assert lib.amoe_gate_grad(5, p, p, p, 4, 2, 8, None) == EINVAL
     assert lib.amoe_row_abs_max(_abi.AMOE_F32, p, 4, 8, 16, p, None) == EINVAL          # ldx < K
     assert lib.amoe_weight_abs_max(_abi.AMOE_F32, p, 2, 8, 16, 3, p, None) == EINVAL   # cols is 1 or N
+    # weight modifier / clip
+    F = _abi.AMOE_F32
+    assert lib.amoe_modify_weight(F, p, 2, 8, 16, p, 3, 14.0, 0.0, None, 1, 0, None, p, None) == EINVAL    # wmax cols
+    assert lib.amoe_modify_weight(F, p, 2, 8, 16, None, 1, 14.0, 0.0, None, 1, 0, None, p, None) == ENULL
+    assert lib.amoe_modify_weight(F, p, 2, 8, 16, p, 1, 14.0, 0.1, p + 2, 1, 0, None, p, None) == EALIGN
+    assert lib.amoe_modify_weight(3, p, 2, 8, 16, p, 1, 14.0, 0.1, None, 1, 0, None, p, None) == EINVAL
+    assert lib.amoe_weight_std_workspace(2, 8, 16, 1) > 0 and lib.amoe_weight_std_workspace(2, 8, 16, 16) > 0
+    assert lib.amoe_weight_std(F, p, 2, 8, 16, 1, p, None, 0, None) == ENULL                # no workspace
+    assert lib.amoe_weight_std(F, p, 2, 8, 16, 1, p, p, 8, None) == EWORKSPACE
+    assert lib.amoe_weight_std(F, p, 0, 8, 16, 1, p, p, 4096, None) == EINVAL
+    assert lib.amoe_clamp_weights(F, p, 2, 8, 16, None, 1, None) == ENULL
+    assert lib.amoe_clamp_weights(F, p, 2, 8, 16, p, 5, None) == EINVAL
+    # router epilogue
+    assert lib.amoe_select_workspace(100, 64) >= 4 * 64
+    assert lib.amoe_select_fwd(F, p, 8, 16, 17, p, p, None, None, None, 0, None) == EINVAL      # k > E
+    assert lib.amoe_select_fwd(F, p, 8, 1024, 2, p, p, None, None, None, 0, None) == EUNSUPPORTED
+    assert lib.amoe_select_fwd(F, p, 8, 16, 2, p, None, None, None, None, 0, None) == ENULL
+    assert lib.amoe_select_fwd(F, p, 8, 16, 2, p, p, p, None, None, 0, None) == EINVAL          # reg without reg_c
+    assert lib.amoe_select_fwd(F, p, 8, 16, 2, p, p, p, p, p, 4, None) == EWORKSPACE
+    assert lib.amoe_select_fwd(F, p, 0, 16, 2, p, p, None, None, None, 0, None) == 0            # no rows: nothing to do
+    assert lib.amoe_select_bwd(F, p, 8, 16, 2, None, p, None, None, p, None) == ENULL           # grad_val needs the ids
+    assert lib.amoe_select_bwd(F, p, 8, 16, 2, p, p, p, None, p, None) == EINVAL                # reg_c without grad_reg
     for rc in (EINVAL, ENULL, ESHAPE, EALIGN, EWORKSPACE, EUNSUPPORTED):
         assert len(lib.amoe_strerror(rc)) > 0
