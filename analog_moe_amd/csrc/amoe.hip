@@ -222,7 +222,8 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   p.out_stage = aligned(a->out, 16) && (a->ldo % CH == 0);
   p.noise_vec = a->noise && aligned(a->noise, 16) && (a->ldnoise % 4 == 0) && (a->noise_tile_stride % 4 == 0);
   const long long lim = 1LL << 31;
-  p.buf_ok = (long long)a->n_in_rows * a->ldx * (long long)es < lim &&
+  // (n_in_rows == 0: the caller does not state the rows of x, so nothing bounds its extent)
+  p.buf_ok = a->n_in_rows > 0 && (long long)a->n_in_rows * a->ldx * (long long)es < lim &&
              ((long long)a->K * a->w_stride_k + (long long)a->N * a->w_stride_n) * (long long)es < lim;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;

@@ -20,17 +20,28 @@ namespace amoe {
 
 enum { MODE_FWD = 0, MODE_FWD_SPLIT = 1, MODE_BWDX = 2 };
 
-// DAC code of a value already clamped to +-r: round((x / r) / res) to nearest even.  fp32 operands take the two
-// correctly rounded divisions of the reference's tensor expression (cvmm.py:150-167), so their codes are
-// bit-identical to it.  bf16 operands take one multiplication by kq = (1 / r) * (1 / res): the gathered rows
-// pass this stage once per block of output columns, and at ten instructions per element it held the vector
-// ALU longer than the matrix instructions hold the matrix pipe (forward up-projection 0.25 -> 0.21 ms).  The
-// product is within 2e-7 (relative) of the quotient, so a code differs, by one step, only for a value that
-// close to a rounding tie -- far inside the tolerance of the bf16 path.
+// DAC code of a value already clamped to +-r: round((x / r) / res) to nearest even, bit-identical to the two
+// correctly rounded divisions of the reference's tensor expression (cvmm.py:150-167).  fp32 operands take the two
+// divisions.  bf16 operands -- whose gathered rows pass this stage once per block of output columns, where ten
+// instructions per element held the vector ALU longer than the matrix instructions hold the matrix pipe -- take one
+// multiplication by kq = (1 / r) * (1 / res); the product is within 6 * 2^-24 (relative) of the double-rounded
+// quotient, so the two can only round differently when the product lies within 6 * 2^-24 * (1 / res + 1) of a
+// half-integer.  dac_code() tracks the largest distance from the rounded code it has seen; when that exceeds
+// dac_tie_margin(1 / res) the caller redoes its values with dac_code_exact (one chunk in ten thousand for 8 bits).
+__device__ __forceinline__ float dac_tie_margin(float resinv) { return 0.5f - 4.0e-7f * (resinv + 1.0f); }
+__device__ __forceinline__ float dac_code_exact(float x, float r, float rinv, float res, float resinv) {
+  return rintf(div_by(div_by(x, r, rinv), res, resinv));
+}
 template <bool IS_BF16>
-__device__ __forceinline__ float dac_code(float x, float r, float rinv, float res, float resinv, float kq) {
-  if constexpr (IS_BF16) return rintf(x * kq);
-  else return rintf(div_by(div_by(x, r, rinv), res, resinv));
+__device__ __forceinline__ float dac_code(float x, float r, float rinv, float res, float resinv, float kq,
+                                          float& tie_dist) {
+  if constexpr (IS_BF16) {
+    const float q = x * kq, c = rintf(q);
+    tie_dist = fmaxf(tie_dist, fabsf(q - c));
+    return c;
+  } else {
+    return dac_code_exact(x, r, rinv, res, resinv);
+  }
 }
 
 struct RowsParams {
@@ -175,6 +186,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
   const bool gen_noise = FWD && p.noise == nullptr && p.noise_std > 0.f;
   const uint64_t seed = p.seed + ((gen_noise && p.seed_dev != nullptr) ? *p.seed_dev : 0);
   const float inv_res = quant ? 1.0f / p.inp_res : 0.f;
+  const float tie_margin = dac_tie_margin(inv_res);
   const bool use_ir_bw = !FWD && p.ir != nullptr;
   // no analog output stage at all: the K-tile result is the accumulator itself
   const bool plain_epi = !codes_mode && p.noise == nullptr && !gen_noise && !adc_clip && !has_amax && !has_ir;
@@ -353,10 +365,17 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
             raw_unpack<T>(ra[i], v);
             const float r = a_ir[i], rinv = a_ir_inv[i];
             const float kq = rinv * inv_res;
+            float tie = 0.f;
+            float xc[CH];
 #pragma unroll
             for (int j = 0; j < CH; j++) {
-              const float c = dac_code<IS_BF16>(clamp_sym(v[j], r), r, rinv, p.inp_res, inv_res, kq);
+              xc[j] = clamp_sym(v[j], r);
+              const float c = dac_code<IS_BF16>(xc[j], r, rinv, p.inp_res, inv_res, kq, tie);
               v[j] = IS_BF16 ? c : c * p.inp_res;
+            }
+            if (IS_BF16 && tie > tie_margin) {      // rare: a product next to a rounding tie
+#pragma unroll
+              for (int j = 0; j < CH; j++) v[j] = dac_code_exact(xc[j], r, rinv, p.inp_res, inv_res);
             }
             if constexpr (IS_BF16) ra[i] = raw_pack_exact_bf16(v);
             else ra[i] = raw_pack<T>(v);
@@ -734,14 +753,21 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
     const float q_r = (FWD && p.xq_out != nullptr) ? p.xq_ir[e] : 1.f;
     const float q_rinv = 1.0f / q_r, q_res = p.xq_inp_res, q_resinv = 1.0f / p.xq_inp_res;
     const float q_kq = q_rinv * q_resinv;
+    const float q_tie_margin = dac_tie_margin(q_resinv);
     auto as_codes = [&](float (&v)[4]) {
+      float tie = 0.f;
+      float xc[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         float x = v[j];
         if constexpr (IS_BF16) x = as_f32((uint32_t)Elem<T>::cvt(x) << 16);
-        x = clamp_sym(x, q_r);
-        const float c = dac_code<IS_BF16>(x, q_r, q_rinv, q_res, q_resinv, q_kq);
+        xc[j] = clamp_sym(x, q_r);
+        const float c = dac_code<IS_BF16>(xc[j], q_r, q_rinv, q_res, q_resinv, q_kq, tie);
         v[j] = IS_BF16 ? c : c * q_res;
+      }
+      if (IS_BF16 && tie > q_tie_margin) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = dac_code_exact(xc[j], q_r, q_rinv, q_res, q_resinv);
       }
     };
     const int n_out = (FWD && p.xq_out != nullptr) ? 2 : 1;

@@ -74,7 +74,9 @@ typedef struct amoe_fwd_args {
   int32_t dtype;                 /* AMOE_F32 / AMOE_BF16: type of x, w, out */
   int32_t M, N, K, E;            /* sorted rows, output features, input features, experts */
   int32_t n_in_rows, n_out_rows; /* rows of x / of out (indices are checked against nothing
-                                    on the device; the caller guarantees the ranges) */
+                                    on the device; the caller guarantees the ranges).
+                                    n_in_rows == 0 = unknown: 64-bit addressing of x, as
+                                    n_x_rows == 0 in amoe_bwd_w_args */
   const void* x;   int64_t ldx;                       /* [n_in_rows, K], row stride ldx */
   const void* w;   int64_t w_stride_e, w_stride_k, w_stride_n; /* [E, K, N] view; one of
                                     w_stride_n / w_stride_k must be 1 (cvmm.py:839 passes a

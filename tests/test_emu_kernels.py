@@ -126,6 +126,15 @@ def test_generated_noise_matches_counter_oracle(emu_ops):
     assert (got["z"] - clean["z"]).abs().max() > 1e-3
 
 
+@pytest.mark.parametrize("split", [False, True])
+def test_generated_noise_interior_bf16(emu_ops, split):
+    util.check_generated_noise_interior(emu_ops, split=split, T=70)
+
+
+def test_bf16_dac_codes_next_to_rounding_ties(emu_ops):
+    util.check_bf16_dac_codes_near_ties(emu_ops)
+
+
 def test_companions(emu_ops):
     pr = util.make_problem(11, T=30, D=70, E=5, F=20, k=2)
     x = pr["x"]

@@ -125,6 +125,20 @@ def test_generated_noise_matches_counter_oracle(ops):
     assert util.rel_err(got["y"].cpu().numpy(), cont.y) < 1e-4
 
 
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_generated_noise_interior(ops, dtype, split):
+    """The output stage the benchmark times (edge-free tiles, bf16 codes, noise drawn in the kernel, ADC, one
+    max |W| per expert, per-expert input ranges; with and without the K-tile split) against the oracle."""
+    print("generated noise, interior tiles", dtype, "split" if split else "one tile", flush=True)
+    print(util.check_generated_noise_interior(ops, device="cuda", dtype=dtype, split=split, T=1500))
+
+
+def test_bf16_dac_codes_next_to_rounding_ties(ops):
+    print("bf16 DAC codes next to rounding ties", flush=True)
+    util.check_bf16_dac_codes_near_ties(ops, device="cuda", T=960)
+
+
 def test_companions(ops):
     pr = _to(util.make_problem(11, T=300, D=70, E=5, F=20, k=2))
     x = pr["x"]

@@ -313,6 +313,128 @@ def test_ir_grad_closed_form_and_special_cases():
     np.testing.assert_array_equal(b2.ir_grad, b.ir_grad)   # too many inputs clip: no decay term
 
 
+# ---- K-tile split in the backward: per-tile clip mask, per-tile input-range gradient (cvmm.py:848-881 per tile)
+TILES_UP, TILES_DN = [0, 40, 90, 128], [0, 24, 64]          # uneven tiles of D = 128 and F = 64
+
+
+def _surrogate_layer_tiled(x, keys, values, idx, gate, ir_up, ir_dn):
+    """The surrogate above with the contraction cut into K-tiles: every tile clamps its slice of the input
+    against its own range, multiplies its slice of the weights, and the tile results are added.  ir_up [E, 3],
+    ir_dn [E, 2]; autograd supplies every gradient, including those of the ranges."""
+    T, k = idx.shape
+    y = torch.zeros(T, values.shape[2])
+    for t in range(T):
+        for h in range(k):
+            e = int(idx[t, h])
+            p = 0
+            for j in range(len(TILES_UP) - 1):
+                lo, hi = TILES_UP[j], TILES_UP[j + 1]
+                r = ir_up[e, j]
+                p = p + torch.minimum(torch.maximum(x[t, lo:hi], -r), r) @ keys[e, lo:hi]
+            p = torch.relu(p)
+            z = 0
+            for j in range(len(TILES_DN) - 1):
+                lo, hi = TILES_DN[j], TILES_DN[j + 1]
+                r = ir_dn[e, j]
+                z = z + torch.minimum(torch.maximum(p[lo:hi], -r), r) @ values[e, lo:hi]
+            y[t] = y[t] + gate[t, h] * z
+    return y
+
+
+def test_tiled_backward_matches_autograd_of_tiled_surrogate():
+    """Pins the multi-tile branch of cvmm_backward / cvmm_bwd_w: clip mask and clipped weight-gradient operand
+    per K-tile on both projections, through grad_x, both weight gradients and the gate gradient.  (The
+    input-range gradient of the reference is not the autograd gradient of a clamp -- it keeps one sign only,
+    cvmm.py:863-865 -- so the brute force below pins it.)"""
+    x, keys, values, idx, gate = _problem(12, T=50)
+    x.requires_grad_(); keys.requires_grad_(); values.requires_grad_(); gate = gate.detach().requires_grad_()
+    g = torch.Generator().manual_seed(5)
+    ir_up = (torch.rand(4, 3, generator=g) * 1.5 + 0.4)
+    ir_dn = (torch.rand(4, 2, generator=g) * 0.8 + 0.2)
+    y = _surrogate_layer_tiled(x, keys, values, idx, gate, ir_up, ir_dn)
+    dy = torch.randn(y.shape, generator=torch.Generator().manual_seed(1))
+    (y * dy).sum().backward()
+    ir = np.zeros((2, 4, 3), np.float32)
+    ir[0] = ir_up.numpy()
+    ir[1, :, :2] = ir_dn.numpy()
+    r = O.layer_fwd_bwd(x.detach().numpy(), keys.detach().numpy(), values.detach().numpy(), idx.numpy(),
+                        gate.detach().numpy(), ir, dy.numpy(), gradient_relative=False,
+                        bounds_up=TILES_UP, bounds_down=TILES_DN)
+    np.testing.assert_allclose(r.y, y.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_values, values.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_keys, keys.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_x, x.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r.grad_gate, gate.grad.numpy(), rtol=1e-4, atol=1e-5)
+    # the masks did something on every tile of both projections
+    xs = x.detach().numpy()
+    for j in range(3):
+        assert (np.abs(xs[:, TILES_UP[j]:TILES_UP[j + 1]]) >= ir_up.numpy()[:, j].min()).any()
+
+
+@pytest.mark.parametrize("proj", ["up", "down"])
+def test_tiled_ir_grad_brute_force(proj):
+    """cvmm.py:848-870 per K-tile, element by element, on both call shapes of CVMM.backward: the
+    up-projection (x [T, K] gathered by perm // k, no gate) and the down-projection (x [M, K] gathered by
+    perm, gate-scaled gradient), three uneven tiles, relative scaling and the decay rule."""
+    x, keys, values, idx, gate = _problem(13, T=40)
+    E, k = 4, 2
+    s = O.prepare_sel(idx.numpy(), E, k)
+    rng = RNG(3)
+    if proj == "up":
+        W, xin, bounds = keys.numpy(), x.numpy(), TILES_UP
+        g = rng.standard_normal((80, 64)).astype(np.float32)
+        sel_index, out_index, gt, z = s.in_index, s.perm, None, None
+    else:
+        W, bounds = values.numpy(), [0, 10, 33, 64]
+        xin = np.maximum(rng.standard_normal((80, 64)), 0).astype(np.float32)
+        g = rng.standard_normal((40, 128)).astype(np.float32)
+        sel_index, out_index, gt = s.perm, None, gate.numpy()
+        z = rng.standard_normal((80, 128)).astype(np.float32)
+    nt = len(bounds) - 1
+    irv = rng.uniform(0.3, 1.4, size=(E, nt)).astype(np.float32)
+    ir = irv[s.sel_sorted]
+    kw = dict(k=k, gradient_relative=True, gradient_scale=0.25, bounds=bounds, relu_mask=(proj == "down"))
+    b = O.cvmm_backward(g, xin, W, s.sel_sorted, sel_index, out_index, gt, ir, z, **kw)
+    W64 = W.astype(np.float64)
+    want = np.zeros((80, nt))
+    want_full = np.zeros((80, W.shape[1]))
+    n_not_clip = 0
+    for j in range(80):
+        e, row = int(s.sel_sorted[j]), int(sel_index[j])
+        o = int(s.perm[j])                               # flat (token, head) position = output row
+        grow = g[o // k] if proj == "down" else g[o]
+        scale = float(gt.reshape(-1)[o]) if proj == "down" else 1.0
+        G = np.float32(grow.astype(np.float64) @ W64[e].T).astype(np.float64)
+        for t in range(nt):
+            acc = 0.0
+            for n in range(bounds[t], bounds[t + 1]):
+                xv = float(xin[row, n])
+                gs = float(np.float32(G[n] * scale))
+                if xv >= irv[e, t]:
+                    acc += min(gs, 0.0)
+                if xv <= -irv[e, t]:
+                    acc -= max(gs, 0.0)
+                keep = abs(xv) < irv[e, t]
+                n_not_clip += keep
+                v = G[n] * keep
+                if proj == "down":
+                    v = v * (xv > 0)
+                want_full[o if proj == "up" else row, n] = v * scale
+            want[j, t] = acc * irv[e, t] * 0.25
+    np.testing.assert_allclose(b.ir_grad, want, rtol=1e-4, atol=1e-5)
+    assert (np.abs(want) > 0).any(axis=0).all()          # every tile contributes
+    np.testing.assert_allclose(b.grad_x_full, want_full, rtol=1e-4, atol=1e-5)
+    # decay: added per tile when the un-clipped share of ALL elements exceeds the threshold (cvmm.py:872-878)
+    pct = n_not_clip / (80 * W.shape[1])
+    lo_thr, hi_thr = pct - 0.01, pct + 0.01
+    bd = O.cvmm_backward(g, xin, W, s.sel_sorted, sel_index, out_index, gt, ir, z, decay=0.02,
+                         input_min_percentage=lo_thr, **kw)
+    np.testing.assert_allclose(bd.ir_grad, want + 0.02 * ir, rtol=1e-4, atol=1e-5)
+    bn = O.cvmm_backward(g, xin, W, s.sel_sorted, sel_index, out_index, gt, ir, z, decay=0.02,
+                         input_min_percentage=hi_thr, **kw)
+    np.testing.assert_array_equal(bn.ir_grad, b.ir_grad)
+
+
 def test_bwd_w_empty_expert_is_zero_and_bf16_rounds():
     x, keys, _, idx, _ = _problem(10, T=30, E=4)
     idx = idx.clamp(max=2)                                   # expert 3 gets nothing
