@@ -83,7 +83,7 @@ class CVMM(torch.autograd.Function):
         ext = ext or AnalogExt()
         E, K, N = keys.shape
         if torch.is_autocast_enabled():
-            dt = torch.get_autocast_gpu_dtype()
+            dt = torch.get_autocast_dtype("cuda")
             if dt != torch.bfloat16:
                 raise RuntimeError("the CVMM kernels autocast to bfloat16 only")
             x, keys_op = x.to(dt), keys.to(dt)

@@ -254,11 +254,13 @@ class AnalogLinear(nn.Module):
             bir = self.input_range.reshape(1, self.n_tiles).expand(x2.shape[0], self.n_tiles)
         w = self.weight.t().unsqueeze(0)                               # [1, in, out]: a transposed view
         modified = w
+        drew = False                                   # a launch of this forward read the device seed word
         if (self.training or self.rpu_config.modifier.enable_during_test) and \
                 enum_name(self.rpu_config.modifier.type) not in ("NONE", "COPY"):
             modified = AnalogSigmaMoELayer.modify_weight(
                 w, self.rpu_config.modifier, injected=self.noise_mode == "injected", seed_dev=self.noise_counter,
                 seed=None if self.noise_mode == "injected" else self._seed() ^ _MODIFIER_ROUTER_SEED)
+            drew = self.noise_mode != "injected"
         ext = AnalogExt(offsets=sel.offsets, bounds=self.bounds,
                         out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
                         out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
@@ -274,6 +276,8 @@ class AnalogLinear(nn.Module):
                 * fwd.out_noise * ext.wmax[0]
         y = CVMM.apply(x2, sel.sel_index, sel.sel, modified, -1.0 if perfect else kernel_inp_res(fwd.inp_res), bir,
                        None, None, out_noise, irp, fwd, ext)
+        if self.noise_counter is not None and (drew or ext.noise_seed_dev is not None):
+            self.noise_counter.add_(1)                 # the next forward (or graph replay) draws anew
         return y.view(*x.shape[:-1], self.out_features)
 
     @torch.no_grad()
@@ -594,8 +598,10 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         perfect = self._io_perfect()
         inp_res = -1.0 if perfect else kernel_inp_res(fwd.inp_res)
         modified = weights
+        drew = False                                   # a launch of this call read the device seed word
         if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
             modified = self._modified(weights, is_down=not is_up)
+            drew = self.noise_mode != "injected"
         ext = AnalogExt(offsets=sel_indices.offsets, bounds=bounds,
                         out_bound=-1.0 if perfect else float(getattr(fwd, "out_bound", -1)),
                         out_res=-1.0 if perfect else float(getattr(fwd, "out_res", -1)))
@@ -613,8 +619,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         res = CVMM.apply(inputs, sel_indices.sel_index, sel_indices.sel, modified, inp_res, bir,
                          sel_indices.out_index, sel_indices.reduction_weight, out_noise,
                          self.rpu_config.pre_post.input_range, fwd, ext)
-        if ext.noise_seed_dev is not None:
-            ext.noise_seed_dev.add_(1)
+        if self.noise_counter is not None and (drew or ext.noise_seed_dev is not None):
+            self.noise_counter.add_(1)                 # output noise or a weight modifier drew from it
         return res
 
     # -- fused path ---------------------------------------------------------------------------------------
@@ -652,7 +658,9 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             cfg.noise_up = torch.randn(ntu, M, self.expert_size, device=x.device) * fwd.out_noise * wu[flat]
             cfg.noise_down = torch.randn(ntd, M, self.v_dim, device=x.device) * fwd.out_noise * wd[flat]
         keys, values = self.keys, self.values
+        drew = False
         if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
+            drew = self.noise_mode != "injected"
             # the output noise and the ADC keep following the max |W| of the unmodified weights
             # (moe_layer_aihwkit_lightning.py:458-489)
             if noisy or cfg.out_bound > 0:
@@ -660,11 +668,17 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
                 cfg.wmax_down = torch.ops.amoe.weight_abs_max(values.detach(), cfg.noise_per_channel)
             keys, values = self._modified(keys, is_down=False), self._modified(values, is_down=True)
         lead = x.shape[:-1]
+        if torch.is_autocast_enabled():            # as CVMM.forward does (cvmm.py:716): compute in the autocast type
+            dt = torch.get_autocast_dtype("cuda")
+            if dt != torch.bfloat16:
+                raise MoEConifgError("the CVMM kernels autocast to bfloat16 only")
+            x = x.to(dt)
         y = moe_ffn(x.reshape(-1, x.shape[-1]), keys.to(x.dtype), values.to(x.dtype),
                     self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
                     sel_idx.reshape(-1, self.n_heads), cfg)
-        if cfg.noise_seed_dev is not None:
-            cfg.noise_seed_dev.add_(2)             # the two projections used seed + 0 and seed + 1
+        if self.noise_counter is not None and (drew or cfg.noise_seed_dev is not None):
+            self.noise_counter.add_(2)             # the two projections used seed + 0 and seed + 1; a weight
+                                                   # modifier alone (no output noise) must see a new word too
         y = y.view(*lead, self.v_dim)
         if self.o_bias is not None:
             y = y + self.o_bias

@@ -423,6 +423,71 @@ def test_weight_modifier_types_run(kind):
     assert layer.keys.grad is not None and torch.isfinite(layer.keys.grad).all() and layer.keys.grad.abs().sum() > 0
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_device_seed_word_advances_for_a_weight_modifier_alone(fused):
+    """With the device seed word, an ADD_NORMAL weight modifier and NO output noise, every forward -- and every
+    replay of a captured forward -- perturbs the weights differently: the word moves whenever a launch read it."""
+    from analog_moe_amd import config as cfgmod
+    mods = {} if fused else {"activation": torch.nn.functional.gelu}
+    layer = _layer(cfgmod, mods, out_noise=0.0)
+    layer.rpu_config.modifier.type = cfgmod.WeightModifierType.ADD_NORMAL
+    layer.rpu_config.modifier.std_dev = 0.2
+    assert layer._fusable() == fused
+    layer.train()
+    word = layer.use_device_noise_counter()
+    x = torch.randn(64, 128, device="cuda")
+    sel_val, sel_idx, _ = layer.select(x)
+    with torch.no_grad():
+        y0 = layer.forward_selected(x, sel_val, sel_idx).clone()
+        w0 = int(word.item())
+        y1 = layer.forward_selected(x, sel_val, sel_idx).clone()
+        w1 = int(word.item())
+    assert w0 > 0 and w1 > w0 and not torch.equal(y0, y1)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            layer.forward_selected(x, sel_val, sel_idx)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = layer.forward_selected(x, sel_val, sel_idx)
+        outs = []
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            outs.append(y_static.clone())
+            assert np.isfinite(torch.randn(1 << 14, device="cuda").sum().item())     # eager work in between
+    assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
+    # eval without enable_during_test: no modifier, nothing reads the word, it stays
+    layer.eval()
+    before = int(word.item())
+    with torch.no_grad():
+        layer.forward_selected(x, sel_val, sel_idx)
+    assert int(word.item()) == before
+
+
+def test_autocast_fused_and_composed_paths_agree():
+    """Under torch.autocast(bfloat16) both layer paths compute in bf16 and return bf16 (cvmm.py:716 makes the
+    autocast type the output type), from fp32 inputs and fp32 parameters; float16 autocast is refused."""
+    from analog_moe_amd import config as cfgmod
+    from analog_moe_amd.moe_layer import MoEConifgError
+    fused = _layer(cfgmod, {})
+    comp = _layer(cfgmod, {"activation": lambda t: torch.relu(t)})
+    comp.load_state_dict(fused.state_dict())
+    assert fused._fusable() and not comp._fusable()
+    x = torch.randn(96, 128, device="cuda")
+    sel_val, sel_idx, _ = fused.select(x)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        a = fused.forward_selected(x, sel_val, sel_idx)
+        b = comp.forward_selected(x, sel_val, sel_idx)
+    assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16
+    assert util.rel_err(util.np32(a), util.np32(b)) < 2e-2
+    with torch.autocast("cuda", dtype=torch.float16):
+        with pytest.raises((MoEConifgError, RuntimeError), match="bfloat16"):
+            fused.forward_selected(x, sel_val, sel_idx)
+
+
 @pytest.mark.parametrize("kind", ["LAYER_GAUSSIAN", "LAYER_GAUSSIAN_PER_CHANNEL", "NONE"])
 def test_clip_types_run(kind):
     """test_moe_layer_aihwkit_lightning.py:287-323, with the bound checked (sigma x std over the expert's
