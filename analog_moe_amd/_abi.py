@@ -66,6 +66,8 @@ PROTOTYPES = {
     "amoe_strerror": (C.c_char_p, [C.c_int]),
     "amoe_prepare_sel_workspace": (SZ, [I64, I32]),
     "amoe_prepare_sel": (C.c_int, [P, I32, I64, I32, I32, P, P, P, P, P, P, SZ, P]),
+    "amoe_noalloc_scratch_bytes": (SZ, []),
+    "amoe_prepare_sel_noalloc": (C.c_int, [P, I32, I64, I32, I32, P, P, P, P, P, P]),
     "amoe_offsets_from_sorted": (C.c_int, [P, I64, I32, P, P]),
     "amoe_cvmm_fwd": (C.c_int, [C.POINTER(FwdArgs), P]),
     "amoe_bwd_w_workspace": (SZ, [C.POINTER(BwdWArgs)]),

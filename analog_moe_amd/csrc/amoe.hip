@@ -1,6 +1,8 @@
 // C ABI of libamoe: argument checks on the host, then kernel launches on the caller's stream.
 #include <amoe.h>
 
+#include <atomic>
+
 #include "gemm_rows.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
@@ -107,7 +109,7 @@ const char* amoe_strerror(int rc) {
     case AMOE_ENULL: return "required pointer is NULL";
     case AMOE_ESHAPE: return "inconsistent sizes";
     case AMOE_EALIGN: return "pointer not aligned to 4 bytes";
-    case AMOE_EWORKSPACE: return "workspace too small";
+    case AMOE_EWORKSPACE: return "workspace too small (or the call exceeds the library's own scratch array)";
     case AMOE_EUNSUPPORTED: return "not supported by this build";
     default: return rc > 0 ? "HIP launch error" : "unknown error";
   }
@@ -153,6 +155,54 @@ int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, 
     if (int rc = launch_rc()) return rc;
   }
   return AMOE_OK;
+}
+
+// ---- selection without any allocation: the unit histograms live in a device array of the library ----------
+}  // extern "C"
+
+// One copy per GPU the library runs on, held until the process ends.  In host code the array's NAME is only a
+// stand-in for the symbol, not a device address: the device address is asked for once per device and kept.
+static __device__ __align__(256) unsigned char scratch[AMOE_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int scratch_address(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return AMOE_EUNSUPPORTED;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (ptr == nullptr) return AMOE_EUNSUPPORTED;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // every thread would store the same address
+  }
+  *out = ptr;
+  return AMOE_OK;
+}
+}  // namespace
+
+extern "C" {
+
+size_t amoe_noalloc_scratch_bytes(void) { return AMOE_NOALLOC_SCRATCH_BYTES; }
+
+int amoe_prepare_sel_noalloc(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, int32_t k,
+                             int32_t* sel_sorted, int32_t* perm, int32_t* in_index, int32_t* offsets,
+                             int32_t* bad_flag, void* stream) {
+  if (M < 0 || M > 0x7fffffffLL || E < 1 || k < 1) return AMOE_EINVAL;
+  if (E > kSelMaxExperts) return AMOE_EUNSUPPORTED;
+  // the histograms of this call must fit the library's array; nothing is allocated to make room
+  if (amoe_prepare_sel_workspace(M, E) > (size_t)AMOE_NOALLOC_SCRATCH_BYTES) return AMOE_EWORKSPACE;
+  void* ws = nullptr;
+  if (int rc = scratch_address(&ws)) return rc;
+  // every unit's histogram row is written by the first pass before anything reads it, so what the previous
+  // call left in the array does not matter and nothing has to be cleared
+  return amoe_prepare_sel(sel, sel_is_i64, M, E, k, sel_sorted, perm, in_index, offsets, bad_flag, ws,
+                          (size_t)AMOE_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, int32_t* offsets, void* stream) {

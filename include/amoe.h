@@ -55,6 +55,19 @@ int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, 
                      int32_t* sel_sorted, int32_t* perm, int32_t* in_index, int32_t* offsets,
                      int32_t* bad_flag, void* workspace, size_t workspace_bytes, void* stream);
 
+/* amoe_prepare_sel for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same selection, bit for bit, without a workspace
+ * argument.  No counterpart in the reference.  The unit histograms live in a device array inside the library
+ * (AMOE_NOALLOC_SCRATCH_BYTES, one copy per GPU the library is used on, held until the process ends); the call
+ * allocates and frees nothing.  A call whose amoe_prepare_sel_workspace(M, E) exceeds that size is rejected with
+ * AMOE_EWORKSPACE (nothing launched).  All calls on one GPU share the array: calls that overlap on one GPU
+ * (different streams, different threads) race; calls on one stream are ordered and safe. */
+#define AMOE_NOALLOC_SCRATCH_BYTES (2u << 20)
+size_t amoe_noalloc_scratch_bytes(void);
+int amoe_prepare_sel_noalloc(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, int32_t k,
+                             int32_t* sel_sorted, int32_t* perm, int32_t* in_index, int32_t* offsets,
+                             int32_t* bad_flag, void* stream);
+
 /* offsets[E+1] from an already sorted id vector, for callers that arrive with the
  * reference's own CVMMSel (cvmm.py:19-28), which carries no offsets. */
 int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, int32_t* offsets,

@@ -35,6 +35,10 @@ inline hipError_t hipGetLastError() { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emu"; }
 enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 0 };
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+// a "device" array is ordinary host memory here, and its address is the symbol's own
+#define __align__(n) __attribute__((aligned(n)))
+#define HIP_SYMBOL(x) (&(x))
+template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; return hipSuccess; }
 // a 3-CU device: the persistent kernels then run few workgroups with several work items each
 inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 3; return hipSuccess; }
 
