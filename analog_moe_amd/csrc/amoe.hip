@@ -228,7 +228,6 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   const bool gen_noise = a->noise == nullptr && a->noise_std > 0.f;
   const bool adc = a->out_bound > 0.f;
   if ((gen_noise || adc) && (!a->wmax || (a->wmax_cols != 1 && a->wmax_cols != a->N))) return AMOE_ESHAPE;
-  if (gen_noise && (a->N % 2)) return AMOE_EUNSUPPORTED;
   if (a->noise && (a->ldnoise < a->N)) return AMOE_ESHAPE;
   if (a->xq_out && (!a->xq_ir || !(a->xq_inp_res > 0.f))) return AMOE_EINVAL;
   if (a->xq_out && a->ldxq < a->N) return AMOE_ESHAPE;

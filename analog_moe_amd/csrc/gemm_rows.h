@@ -507,6 +507,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
         // max |W| per expert, input range -- as straight-line code: same operations in the same order as the
         // general stage below, without a branch around every 4 values.
         const NoiseKey key = noise_key(seed, t);
+        uint32_t col_key[2];
+#pragma unroll
+        for (int fi = 0; fi < 2; fi++) col_key[fi] = noise_col_key(key, (uint32_t)(c0 + wc * 64 + fi * 32 + l32));
+        const float u_nzs = u_nz * kNoiseScale;
 #pragma unroll
         for (int ti = 0; ti < 2; ti++) {
           const int rl = wr * 64 + ti * 32 + l32;
@@ -517,16 +521,15 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           const uint32_t row_key = noise_row_key(key, (uint32_t)orow);
 #pragma unroll
           for (int fi = 0; fi < 2; fi++) {
+            // the block's noise: one 8-bit matrix instruction (same slot layout as acc[fi][ti])
+            const i32x16 zi = noise_block(row_key, col_key[fi], (uint32_t)(c0 + wc * 64 + fi * 32) >> 5,
+                                          (uint32_t)(row0 + wr * 64 + ti * 32), lh);
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-              const int col = c0 + wc * 64 + fi * 32 + 8 * q + 4 * lh;
-              float z[4];
-              noise_pair(key, row_key, (uint32_t)(col >> 1), z[0], z[1]);
-              noise_pair(key, row_key, (uint32_t)(col >> 1) + 1u, z[2], z[3]);
 #pragma unroll
               for (int j = 0; j < 4; j++) {
                 float v = acc[fi][ti][4 * q + j] * p.inp_res;
-                v += u_nz * z[j];
+                v = fmaf((float)zi[4 * q + j], u_nzs, v);
                 v = clamp_sym(v, u_bound);
                 v = rintf(v * u_q) * u_qinv;
                 v *= ir_r;
@@ -549,6 +552,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
           const uint32_t row_key = gen_noise ? noise_row_key(key, (uint32_t)orow) : 0u;
 #pragma unroll
           for (int fi = 0; fi < 2; fi++) {
+            i32x16 zi;
+            if (gen_noise) {
+              const int cb0 = c0 + wc * 64 + fi * 32;
+              zi = noise_block(row_key, noise_col_key(key, (uint32_t)(cb0 + l32)), (uint32_t)cb0 >> 5,
+                               (uint32_t)(row0 + wr * 64 + ti * 32), lh);
+            }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
               const int cl = wc * 64 + fi * 32 + 8 * q + 4 * lh;
@@ -570,11 +579,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
                 for (int j = 0; j < 4; j++) v[j] += nz[j];
               } else if (gen_noise) {
-                float z[4];
-                noise_pair(key, row_key, (uint32_t)(col >> 1), z[0], z[1]);
-                noise_pair(key, row_key, (uint32_t)(col >> 1) + 1u, z[2], z[3]);
 #pragma unroll
-                for (int j = 0; j < 4; j++) v[j] += (col_uniform ? u_nz : sCol[0][cl + j]) * z[j];
+                for (int j = 0; j < 4; j++)
+                  v[j] = fmaf((float)zi[4 * q + j], (col_uniform ? u_nz : sCol[0][cl + j]) * kNoiseScale, v[j]);
               }
               if (adc_clip && col_uniform) {
 #pragma unroll

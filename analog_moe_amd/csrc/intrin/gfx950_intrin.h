@@ -26,6 +26,16 @@ __device__ __forceinline__ f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c)
                                                  __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// 32x32x32 signed 8-bit product, 32-bit integer accumulate: lane l supplies 16 bytes of row l%32 of each
+// operand (contraction indices 16*(l/32) .. +15); D as for the fp32 tiles.
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+__device__ __forceinline__ i32x16 mfma_i32_32x32x32_i8(u32x4 a, u32x4 b, i32x16 c) {
+  return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), c, 0, 0, 0);
+}
+// (a mod 2^24) * (b mod 2^24) mod 2^32: a full-rate multiply (the 32-bit one runs at a quarter of the rate)
+__device__ __forceinline__ uint32_t mul_u24(uint32_t a, uint32_t b) { return __umul24(a, b); }
+
 __device__ __forceinline__ f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }

@@ -110,7 +110,7 @@ typedef struct amoe_fwd_args {
   const float* noise;            /* [n_tiles, n_out_rows, N] fp32, already scaled, or NULL */
   int64_t noise_tile_stride, ldnoise;
   float noise_std;               /* used when noise == NULL and > 0: generate in the kernel
-                                    noise_std * wmax[e, n] * N(0,1), N even */
+                                    noise_std * wmax[e, n] * N(0,1) */
   uint64_t noise_seed;
   const uint64_t* noise_seed_dev;/* optional device word added to noise_seed when the kernel starts:
                                     a captured graph draws new noise on each replay if the caller

@@ -15,7 +15,10 @@ exists to compare with; the definitions here are this build's own):
 ``tile_bounds`` / the multi-tile path of ``cvmm_fwd`` and ``cvmm_backward``
 (``max_input_size`` splitting), the ADC (``out_bound`` / ``out_res``) stage of
 ``cvmm_fwd``, and ``counter_noise`` (the in-kernel counter-based Gaussian generator,
-which replaces the reference's ``torch.randn`` stream).
+which replaces the reference's ``torch.randn`` stream).  The oracle's own statements of these
+definitions are checked all the same: the multi-tile backward against autograd of a tile-wise surrogate
+and an element-by-element brute force, the tile split and the ADC by their closed-form properties, the
+generator by its statistics.
 
 All reference citations are relative to the reference checkout.
 """
@@ -149,7 +152,9 @@ def adc(c: np.ndarray, wmax_row: np.ndarray, out_bound: float, out_res: float) -
 
 # --------------------------------------------------------------------------------------
 # counter-based Gaussian noise (BUILD-DEFINED; replaces torch.randn of
-# moe_layer_aihwkit_lightning.py:472-477 so that noise can be produced inside the kernel)
+# moe_layer_aihwkit_lightning.py:472-477 so that noise can be produced inside the kernel:
+# the noise of a 32 x 32 block of outputs is a product of two matrices of pseudo-random
+# signed bytes, which the kernel forms with one 8-bit matrix instruction)
 # --------------------------------------------------------------------------------------
 def _fmix32(h: np.ndarray) -> np.ndarray:
     h = h.astype(np.uint32)
@@ -165,9 +170,9 @@ def _u32(v) -> np.ndarray:
     return (np.asarray(v, dtype=np.uint64) & np.uint64(0xFFFFFFFF)).astype(np.uint32)
 
 
-def counter_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.ndarray:
-    """Standard-normal noise for output rows ``rows`` (output-row ids), all ``n_cols``
-    columns, K-tile ``tile``; a pure function of (seed, tile, row, column).
+def box_muller_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.ndarray:
+    """The generator of the weight modifier's normals (``weights_oracle.modifier_normals``): standard-normal
+    values for rows ``rows``, all ``n_cols`` columns, stream ``tile``; a pure function of (seed, tile, row, column).
 
     Columns are paired (2p, 2p+1).  Two 32-bit keys come from the seed halves and the tile.  The
     row gets the key ``fmix32(row ^ ka)``; the pair's word is that key plus ``p * 0x9E3779B9``,
@@ -197,6 +202,60 @@ def counter_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.nda
     out[:, 0::2] = (r * np.cos(ang)).astype(F32)
     out[:, 1::2] = (r * np.sin(ang)).astype(F32)
     return out
+
+
+NOISE_MULTIPLIERS = (0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB, 0x165667, 0xD3A265, 0xFD7047, 0xB55A4F)
+NOISE_SCALE = F32(1.0 / (5.656854249492380195 * 5461.5))     # 1 / (sqrt(32) * std of a product of two bytes)
+
+
+def _noise_words(keys: np.ndarray) -> np.ndarray:
+    """keys [...] uint32 -> [..., 32] signed bytes: the 8 words ``w_j = (key mod 2^24) * c_j + key``,
+    ``w_j ^= w_j >> 15`` with the odd 24-bit multipliers ``NOISE_MULTIPLIERS``, little-endian bytes."""
+    keys = np.asarray(keys, dtype=np.uint32)
+    out = np.empty(keys.shape + (32,), dtype=np.int64)
+    for j in range(8):
+        cj = np.uint64(NOISE_MULTIPLIERS[j])
+        w = _u32((keys & np.uint32(0xFFFFFF)).astype(np.uint64) * cj + keys.astype(np.uint64))
+        w ^= w >> np.uint32(15)
+        for b in range(4):
+            v = ((w >> np.uint32(8 * b)) & np.uint32(0xFF)).astype(np.int64)
+            out[..., 4 * j + b] = np.where(v >= 128, v - 256, v)
+    return out
+
+
+def counter_noise_int(rows: np.ndarray, block_starts: np.ndarray, n_cols: int, tile: int, seed: int) -> np.ndarray:
+    """Integer noise [R, n_cols] for output rows ``rows`` (output-row ids) whose 32-row block starts at sorted
+    position ``block_starts[i]``; K-tile ``tile``.  A pure function of (seed, tile, output row, block start,
+    column): for the 32 x 32 block of a row block and a column block c // 32,
+        z[row][col] = sum_k a[row][k] * b[col][k] - 8
+    with the signed bytes  a[row] = words(fmix32(row ^ ka) ^ (col // 32) * 0x632BE5AB)  and
+    b[col] = words(fmix32(col * 0x9E3779B1 ^ kb) ^ block_start * 0x27D4EB2F); ka, kb are the two 32-bit keys
+    of (seed, tile).  Mean 0, standard deviation 1 / NOISE_SCALE, close to normal (a sum of 32 products)."""
+    rows = _u32(np.asarray(rows, dtype=np.uint64)).reshape(-1)
+    block_starts = _u32(np.asarray(block_starts, dtype=np.uint64)).reshape(-1)
+    s_lo, s_hi = seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF
+    ka = _fmix32(_u32((s_lo ^ 0x9E3779B9) + tile * 0x632BE5AB))
+    kb = _fmix32(_u32((s_hi ^ 0x85EBCA77) + tile * 0x27D4EB2F))
+    row_key = _fmix32(rows ^ ka)                                                     # [R]
+    cols = np.arange(n_cols, dtype=np.uint64)
+    col_key = _fmix32(_u32(cols * np.uint64(0x9E3779B1)) ^ kb)                       # [N]
+    n_cb = (n_cols + 31) // 32
+    out = np.zeros((rows.shape[0], n_cols), dtype=np.int64)
+    ustarts, inv = np.unique(block_starts, return_inverse=True)
+    # b vectors per (block start, column)
+    bkeys = col_key[None, :] ^ _u32(ustarts[:, None].astype(np.uint64) * np.uint64(0x27D4EB2F))
+    bvec = _noise_words(bkeys)                                                       # [S, N, 32]
+    for cb in range(n_cb):
+        c0, c1 = cb * 32, min(cb * 32 + 32, n_cols)
+        akeys = row_key ^ _u32(np.uint64(cb) * np.uint64(0x632BE5AB))
+        avec = _noise_words(akeys)                                                   # [R, 32]
+        out[:, c0:c1] = np.einsum("rk,rck->rc", avec, bvec[inv, c0:c1]) - 8
+    return out
+
+
+def counter_noise(rows: np.ndarray, block_starts: np.ndarray, n_cols: int, tile: int, seed: int) -> np.ndarray:
+    """``counter_noise_int`` scaled to unit variance (fp32)."""
+    return (counter_noise_int(rows, block_starts, n_cols, tile, seed).astype(F32) * NOISE_SCALE).astype(F32)
 
 
 # --------------------------------------------------------------------------------------
@@ -259,8 +318,12 @@ def cvmm_fwd(x, sel_index, sel_sorted, keys, inp_res=-1.0, ir=None, out_index=No
             if noise is not None:
                 c = (c + noise[t, rout, :]).astype(F32)
             elif noise_seed is not None and noise_std > 0:
-                z = counter_noise(rout, N, t, noise_seed)
-                c = (c + (F32(noise_std) * wmax[e][None, :]).astype(F32) * z).astype(F32)
+                # 32-row blocks are counted from the expert's first sorted position
+                starts = pos[0] + (np.arange(len(pos)) // 32) * 32
+                zi = counter_noise_int(rout, starts, N, t, noise_seed).astype(F32)
+                nz = ((F32(noise_std) * wmax[e][None, :]).astype(F32) * NOISE_SCALE).astype(F32)
+                # one fused multiply-add, as the kernel does it (the product is exact in float64)
+                c = (zi.astype(np.float64) * nz.astype(np.float64) + c.astype(np.float64)).astype(F32)
             if out_bound is not None and out_bound > 0:
                 c = adc(c, wmax[e][None, :], out_bound, out_res)
             if amax is not None:

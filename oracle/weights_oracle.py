@@ -14,7 +14,7 @@ third-party ``aihwkit_lightning`` (not in the reference checkout, no version pin
 as ``round(w / res) * res`` with round-half-to-even, which the tests pin only through what any uniform quantiser
 with step ``res`` must satisfy (results are multiples of ``res`` within ``res / 2`` of the input, the largest
 weight maps to itself, the map is idempotent) and through the same expression evaluated by torch.  The normals
-themselves come from ``torch.randn`` in the reference and from ``cvmm_oracle.counter_noise`` here.
+themselves come from ``torch.randn`` in the reference and from ``cvmm_oracle.box_muller_noise`` here.
 """
 from __future__ import annotations
 
@@ -22,7 +22,7 @@ from typing import Optional
 
 import numpy as np
 
-from .cvmm_oracle import F32, _cast, counter_noise
+from .cvmm_oracle import F32, _cast, box_muller_noise
 
 MODIFIER_STREAM = 0x4D4F44      # the "K-tile" id that keeps the modifier's draws apart from the output noise
 
@@ -38,7 +38,7 @@ def assumed_wmax(w: np.ndarray, per_channel: bool) -> np.ndarray:
 def modifier_normals(E: int, K: int, N: int, seed: int) -> np.ndarray:
     """The kernel's own draws: row e*K + k of the counter-based generator, column n."""
     n2 = N + (N & 1)
-    z = counter_noise(np.arange(E * K), n2, MODIFIER_STREAM, seed)
+    z = box_muller_noise(np.arange(E * K), n2, MODIFIER_STREAM, seed)
     return z[:, :N].reshape(E, K, N)
 
 

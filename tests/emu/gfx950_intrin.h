@@ -79,6 +79,31 @@ inline f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c) {
   return c;
 }
 
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+inline i32x16 mfma_i32_32x32x32_i8(u32x4 a, u32x4 b, i32x16 c) {
+  struct Ops { int8_t a[16], b[16]; } mine;
+  std::memcpy(mine.a, &a, 16);
+  std::memcpy(mine.b, &b, 16);
+  EmuWave* w = emu_wave;
+  const int l = lane_id();
+  std::memcpy(w->slot[l], &mine, sizeof(mine));
+  w->bar.arrive_and_wait();
+  const int col = l % 32;
+  for (int i = 0; i < 16; i++) {
+    const int row = 8 * (i / 4) + 4 * (l / 32) + (i % 4);
+    int s = c[i];
+    for (int k = 0; k < 32; k++) {
+      const Ops* pa = (const Ops*)w->slot[row + 32 * (k / 16)];
+      const Ops* pb = (const Ops*)w->slot[col + 32 * (k / 16)];
+      s += (int)pa->a[k % 16] * (int)pb->b[k % 16];
+    }
+    c[i] = s;
+  }
+  w->bar.arrive_and_wait();
+  return c;
+}
+inline uint32_t mul_u24(uint32_t a, uint32_t b) { return (uint32_t)((uint64_t)(a & 0xffffffu) * (uint64_t)(b & 0xffffffu)); }
+
 inline f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
   struct Ops { float a, b; } mine{a, b};
   EmuWave* w = emu_wave;

@@ -225,19 +225,71 @@ def test_adc_off_is_identity_and_on_gives_integer_codes():
 
 
 def test_counter_noise_statistics_and_determinism():
-    rows = np.arange(4096)
-    a = O.counter_noise(rows, 256, 0, 1234)
-    assert np.array_equal(a, O.counter_noise(rows, 256, 0, 1234))
-    assert np.array_equal(a[100:200], O.counter_noise(rows[100:200], 256, 0, 1234))
-    b = O.counter_noise(rows, 256, 1, 1234)
-    c = O.counter_noise(rows, 256, 0, 1235)
-    assert abs(a.mean()) < 5e-3 and abs(a.std() - 1) < 5e-3
+    """The output-noise generator (32 x 32 blocks, each the product of two matrices of pseudo-random signed
+    bytes): a pure function of its arguments, standard normal to the accuracy a sample of a million shows
+    (moments, Kolmogorov distance), uncorrelated between neighbouring rows, columns, blocks, tiles and seeds, and
+    squares only as dependent as the bilinear form makes them (0.012 between entries that share a row or a column of
+    a block for ideal random bytes)."""
+    from scipy import stats as st
+    rows = np.arange(4096) * 7 + 3                       # output rows are scattered ids
+    starts = 11 + (np.arange(4096) // 32) * 32           # 32-row blocks from the expert's first sorted position
+    a = O.counter_noise(rows, starts, 256, 0, 1234)
+    assert a.dtype == np.float32 and a.shape == (4096, 256)
+    assert np.array_equal(a, O.counter_noise(rows, starts, 256, 0, 1234))
+    assert np.array_equal(a[96:200], O.counter_noise(rows[96:200], starts[96:200], 256, 0, 1234))
+    assert np.array_equal(a[:, :70], O.counter_noise(rows, starts, 70, 0, 1234))          # a ragged last block
+    zi = O.counter_noise_int(rows[:64], starts[:64], 64, 0, 1234)
+    assert np.array_equal(zi.astype(np.float32) * O.NOISE_SCALE, a[:64, :64])
+    b = O.counter_noise(rows, starts, 256, 1, 1234)
+    c = O.counter_noise(rows, starts, 256, 0, 1235)
+    d = O.counter_noise(rows, starts + 32, 256, 0, 1234)   # the same output rows in other blocks
+    assert abs(a.mean()) < 4e-3 and abs(a.std() - 1) < 4e-3
     kurt = ((a - a.mean()) ** 4).mean() / a.var() ** 2
-    assert abs(kurt - 3) < 0.05
+    skew = ((a - a.mean()) ** 3).mean() / a.std() ** 3
+    assert abs(kurt - 3) < 0.05 and abs(skew) < 0.01
+    assert st.kstest(a.ravel()[::4], "norm").statistic < 5e-3
+    assert np.abs(a).max() > 4.0                         # tails exist (a sum of 12 uniforms would stop at 6, IH4 at 3.5)
     for other in (b, c):
         assert abs(np.corrcoef(a.ravel(), other.ravel())[0, 1]) < 5e-3
-    assert abs(np.corrcoef(a[:, 0::2].ravel(), a[:, 1::2].ravel())[0, 1]) < 5e-3
-    assert abs(np.corrcoef(a[:-1].ravel(), a[1:].ravel())[0, 1]) < 5e-3
+    assert abs(np.corrcoef(a.ravel(), d.ravel())[0, 1]) < 2e-2
+    for sh in (1, 2, 31, 32, 33):
+        assert abs(np.corrcoef(a[:, :-sh].ravel(), a[:, sh:].ravel())[0, 1]) < 5e-3
+        assert abs(np.corrcoef(a[:-sh].ravel(), a[sh:].ravel())[0, 1]) < 5e-3
+    sq = a.astype(np.float64) ** 2
+    assert abs(np.corrcoef(sq[:, :-1].ravel(), sq[:, 1:].ravel())[0, 1]) < 0.03
+    assert abs(np.corrcoef(sq[:-1].ravel(), sq[1:].ravel())[0, 1]) < 0.03
+    # the energy of a row over 256 columns scatters like that of 256 independent normals (0.088) -- not more than
+    # a quarter above it, as it would if one draw scaled a whole row
+    row_energy = sq.mean(1)
+    assert row_energy.std() < 1.25 * np.sqrt(2 / 256)
+
+
+def test_counter_noise_block_is_a_byte_matrix_product():
+    """Brute force of one block from the definition: words -> signed bytes -> 32-term products."""
+    def fmix(h):
+        h &= 0xFFFFFFFF
+        h ^= h >> 16; h = (h * 0x85EBCA6B) & 0xFFFFFFFF; h ^= h >> 13; h = (h * 0xC2B2AE35) & 0xFFFFFFFF; h ^= h >> 16
+        return h
+
+    def vec(key):
+        out = []
+        for j, cj in enumerate((0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB, 0x165667, 0xD3A265, 0xFD7047, 0xB55A4F)):
+            w = ((key & 0xFFFFFF) * cj + key) & 0xFFFFFFFF
+            w ^= w >> 15
+            for b in range(4):
+                v = (w >> (8 * b)) & 0xFF
+                out.append(v - 256 if v >= 128 else v)
+        return out
+    seed, tile = 0xABCDEF0123456789, 2
+    ka = fmix((((seed & 0xFFFFFFFF) ^ 0x9E3779B9) + tile * 0x632BE5AB) & 0xFFFFFFFF)
+    kb = fmix((((seed >> 32) ^ 0x85EBCA77) + tile * 0x27D4EB2F) & 0xFFFFFFFF)
+    rows, start = [5, 900000, 17], 4096 + 64
+    got = O.counter_noise_int(np.array(rows), np.full(3, start), 40, tile, seed)
+    for i, r in enumerate(rows):
+        for c in (0, 1, 31, 32, 39):
+            a = vec(fmix(r ^ ka) ^ (((c // 32) * 0x632BE5AB) & 0xFFFFFFFF))
+            b = vec(fmix(((c * 0x9E3779B1) & 0xFFFFFFFF) ^ kb) ^ ((start * 0x27D4EB2F) & 0xFFFFFFFF))
+            assert got[i, c] == sum(x * y for x, y in zip(a, b)) - 8
 
 
 # ------------------------------------------------------------------ backward
@@ -586,7 +638,7 @@ def test_modifier_normals_are_standard_and_keyed():
     z = WO.modifier_normals(4, 64, 33, 99)
     assert z.shape == (4, 64, 33) and abs(z.mean()) < 0.03 and abs(z.std() - 1) < 0.03
     assert np.array_equal(z, WO.modifier_normals(4, 64, 33, 99)) and not np.array_equal(z, WO.modifier_normals(4, 64, 33, 100))
-    assert not np.array_equal(z[:, :, :32].reshape(256, 32), O.counter_noise(np.arange(256), 32, 0, 99))
+    assert not np.array_equal(z[:, :, :32].reshape(256, 32), O.box_muller_noise(np.arange(256), 32, 0, 99))
 
 
 # ---------------------------------------------------------------------------------- router epilogue
