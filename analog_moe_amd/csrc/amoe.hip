@@ -4,6 +4,7 @@
 #include <atomic>
 
 #include "gemm_rows.h"
+#include "gemm_fwd256.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
 #include "weight_kernels.h"
@@ -94,6 +95,40 @@ template <typename T, bool W_KC>
 int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
   return rows_all_interior(p, mode, Elem<T>::kBK) ? launch_rows_mode<T, W_KC, true>(p, mode, grid, st)
                                             : launch_rows_mode<T, W_KC, false>(p, mode, grid, st);
+}
+
+// The 128 x 256 forward kernel for the usual training shapes (bf16, every tile interior, per-expert input
+// ranges, one max |W| per expert).  AMOE_EUNSUPPORTED: this launch is not one of them; the general kernel runs.
+template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2>
+int launch_fwd256_as(const RowsParams& p, int grid, hipStream_t st) {
+  auto k = &fwd256_kernel<A_MODE, ANALOG, NOISE, SPLIT2>;
+  hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
+  return launch_rc();
+}
+
+int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st) {
+  if (!rows_all_interior(p, mode, kFBK) || a->N % kFCols) return AMOE_EUNSUPPORTED;
+  if (a->noise != nullptr || a->n_tiles > 2) return AMOE_EUNSUPPORTED;
+  const bool dac = a->ir != nullptr;                 // (interior launches have the range and the quantiser, or neither)
+  if (dac && !a->ir_by_expert) return AMOE_EUNSUPPORTED;
+  const bool adc = a->out_bound > 0.f, noisy = a->noise_std > 0.f;
+  const bool analog = adc && a->out_res > 0.f && a->wmax_cols == 1 && dac;
+  if ((adc || noisy) && !analog) return AMOE_EUNSUPPORTED;
+  if (a->n_tiles == 2 && !(analog && !a->x_is_quantized)) return AMOE_EUNSUPPORTED;
+  p.n_col_blocks = a->N / kFCols;
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
+  if (!dac) return launch_fwd256_as<FA_PLAIN, false, false, false>(p, grid, st);
+  if (!analog)
+    return a->x_is_quantized ? launch_fwd256_as<FA_CODES, false, false, false>(p, grid, st)
+                             : launch_fwd256_as<FA_DAC, false, false, false>(p, grid, st);
+  if (a->x_is_quantized)
+    return noisy ? launch_fwd256_as<FA_CODES, true, true, false>(p, grid, st)
+                 : launch_fwd256_as<FA_CODES, true, false, false>(p, grid, st);
+  if (a->n_tiles == 2)
+    return noisy ? launch_fwd256_as<FA_DAC, true, true, true>(p, grid, st)
+                 : launch_fwd256_as<FA_DAC, true, false, true>(p, grid, st);
+  return noisy ? launch_fwd256_as<FA_DAC, true, true, false>(p, grid, st)
+               : launch_fwd256_as<FA_DAC, true, false, false>(p, grid, st);
 }
 
 }  // namespace
@@ -274,9 +309,13 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   // (n_in_rows == 0: the caller does not state the rows of x, so nothing bounds its extent)
   p.buf_ok = a->n_in_rows > 0 && (long long)a->n_in_rows * a->ldx * (long long)es < lim &&
              ((long long)a->K * a->w_stride_k + (long long)a->N * a->w_stride_n) * (long long)es < lim;
-  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a->dtype == AMOE_BF16 && !w_kc) {
+    const int rc = launch_fwd256(p, mode, a, st);
+    if (rc != AMOE_EUNSUPPORTED) return rc;
+  }
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (a->dtype == AMOE_F32)
     return w_kc ? launch_rows<float, true>(p, mode, grid, st) : launch_rows<float, false>(p, mode, grid, st);
   return w_kc ? launch_rows<uint16_t, true>(p, mode, grid, st) : launch_rows<uint16_t, false>(p, mode, grid, st);

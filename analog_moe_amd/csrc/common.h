@@ -296,21 +296,25 @@ __device__ __forceinline__ void noise_pair(const NoiseKey& key, uint32_t row_key
 // with mean 0 and standard deviation sqrt(32) * 5461.5, approximately normal (excess kurtosis 0.01; entries of a
 // block are uncorrelated, blocks are independent).  One 8-bit matrix instruction per block replaces a hash and a
 // Box-Muller transform per output; what is left per output is one integer-to-float conversion.
-//   a[row] : 8 words  noise_word(row_key ^ (col / 32) * 0x632BE5AB, j),  row_key = fmix32(out_row ^ ka)
-//   b[col] : 8 words  noise_word(col_key ^ block_start * 0x27D4EB2F, j), col_key = fmix32(col * 0x9E3779B1 ^ kb)
+//   a[row] : the 8 words of the key  row_key ^ (col / 32) * 0x632BE5AB,   row_key = fmix32(out_row ^ ka)
+//   b[col] : the 8 words of the key  col_key ^ block_start * 0x27D4EB2F,  col_key = fmix32(col * 0x9E3779B1 ^ kb)
 // (xor, not add: keys that differ by a constant give words that differ by a constant, hence correlated bytes)
 // block_start = sorted position of the block's first row: blocks are the 32-row groups counted from the first
 // sorted position of the expert.  Byte i of word j is contraction index 4 * j + i (any pairing gives the same sum).
 constexpr float kNoiseScale = (float)(1.0 / (5.656854249492380195 * 5461.5));
-// (unrelated odd 24-bit multipliers: words made with multipliers in arithmetic progression are in arithmetic
-// progression themselves, which shows as an excess kurtosis of 0.1)
-__device__ __host__ inline uint32_t noise_const(int j) {
-  constexpr uint32_t c[8] = {0x9E3779u, 0x85EBCBu, 0xC2B2AFu, 0x27D4EBu, 0x165667u, 0xD3A265u, 0xFD7047u, 0xB55A4Fu};
-  return c[j];
-}
+// word j (0 .. 7) of a key's vector: words 0 .. 3 from the key, words 4 .. 7 from key ^ kNoiseHalfKey, each
+// (k mod 2^24) * c_(j mod 4) + k followed by one xor-shift.  (Unrelated odd 24-bit multipliers: with multipliers in
+// arithmetic progression the words are in arithmetic progression too, which shows as an excess kurtosis of 0.1.
+// The four multipliers are the same for every lane, so they live in scalar registers.)
+constexpr uint32_t kNoiseHalfKey = 0x5BD1E995u;
+constexpr uint32_t kNoiseMul0 = 0x9E3779u, kNoiseMul1 = 0x85EBCBu, kNoiseMul2 = 0xC2B2AFu, kNoiseMul3 = 0x27D4EBu;
 __device__ __forceinline__ uint32_t noise_word(uint32_t key, uint32_t cj) {
   uint32_t w = mul_u24(key, cj) + key;
   return w ^ (w >> 15);
+}
+__device__ __forceinline__ u32x4 noise_words(uint32_t key) {
+  return u32x4{noise_word(key, kNoiseMul0), noise_word(key, kNoiseMul1), noise_word(key, kNoiseMul2),
+               noise_word(key, kNoiseMul3)};
 }
 __device__ __forceinline__ uint32_t noise_col_key(const NoiseKey& key, uint32_t col) {
   return fmix32((col * 0x9E3779B1u) ^ key.kb);
@@ -320,15 +324,10 @@ __device__ __forceinline__ uint32_t noise_col_key(const NoiseKey& key, uint32_t 
 // operand is the column side).  half = l / 32 picks the lane's 16 of the 32 contraction indices.
 __device__ __forceinline__ i32x16 noise_block(uint32_t row_key, uint32_t col_key, uint32_t col_block,
                                               uint32_t block_start, int half) {
-  const uint32_t ak = row_key ^ (col_block * 0x632BE5ABu);
-  const uint32_t bk = col_key ^ (block_start * 0x27D4EB2Fu);
-  u32x4 aw, bw;
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const uint32_t cj = half ? noise_const(4 + j) : noise_const(j);
-    aw[j] = noise_word(ak, cj);
-    bw[j] = noise_word(bk, cj);
-  }
+  const uint32_t hk = half ? kNoiseHalfKey : 0u;
+  const uint32_t ak = row_key ^ (col_block * 0x632BE5ABu) ^ hk;
+  const uint32_t bk = col_key ^ (block_start * 0x27D4EB2Fu) ^ hk;
+  const u32x4 aw = noise_words(ak), bw = noise_words(bk);
   i32x16 c;
 #pragma unroll
   for (int i = 0; i < 16; i++) c[i] = -8;

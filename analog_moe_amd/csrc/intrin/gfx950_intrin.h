@@ -36,6 +36,11 @@ __device__ __forceinline__ i32x16 mfma_i32_32x32x32_i8(u32x4 a, u32x4 b, i32x16 
 // (a mod 2^24) * (b mod 2^24) mod 2^32: a full-rate multiply (the 32-bit one runs at a quarter of the rate)
 __device__ __forceinline__ uint32_t mul_u24(uint32_t a, uint32_t b) { return __umul24(a, b); }
 
+// byte `sel` (0..3) of `old` replaced by v converted to an unsigned 8-bit integer (v integral, 0 .. 255 here)
+__device__ __forceinline__ uint32_t cvt_pk_u8_f32(float v, int sel, uint32_t old) {
+  return __builtin_amdgcn_cvt_pk_u8_f32(v, (uint32_t)sel, old);
+}
+
 __device__ __forceinline__ f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }

@@ -204,18 +204,21 @@ def box_muller_noise(rows: np.ndarray, n_cols: int, tile: int, seed: int) -> np.
     return out
 
 
-NOISE_MULTIPLIERS = (0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB, 0x165667, 0xD3A265, 0xFD7047, 0xB55A4F)
+NOISE_MULTIPLIERS = (0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB)
+NOISE_HALF_KEY = 0x5BD1E995
 NOISE_SCALE = F32(1.0 / (5.656854249492380195 * 5461.5))     # 1 / (sqrt(32) * std of a product of two bytes)
 
 
 def _noise_words(keys: np.ndarray) -> np.ndarray:
-    """keys [...] uint32 -> [..., 32] signed bytes: the 8 words ``w_j = (key mod 2^24) * c_j + key``,
-    ``w_j ^= w_j >> 15`` with the odd 24-bit multipliers ``NOISE_MULTIPLIERS``, little-endian bytes."""
+    """keys [...] uint32 -> [..., 32] signed bytes.  Words 0..3 come from the key, words 4..7 from
+    ``key ^ NOISE_HALF_KEY``; word j is ``w = (k mod 2^24) * c_(j mod 4) + k``, ``w ^= w >> 15`` with the odd
+    24-bit multipliers ``NOISE_MULTIPLIERS``; bytes little-endian."""
     keys = np.asarray(keys, dtype=np.uint32)
     out = np.empty(keys.shape + (32,), dtype=np.int64)
     for j in range(8):
-        cj = np.uint64(NOISE_MULTIPLIERS[j])
-        w = _u32((keys & np.uint32(0xFFFFFF)).astype(np.uint64) * cj + keys.astype(np.uint64))
+        k = keys ^ np.uint32(NOISE_HALF_KEY if j >= 4 else 0)
+        cj = np.uint64(NOISE_MULTIPLIERS[j % 4])
+        w = _u32((k & np.uint32(0xFFFFFF)).astype(np.uint64) * cj + k.astype(np.uint64))
         w ^= w >> np.uint32(15)
         for b in range(4):
             v = ((w >> np.uint32(8 * b)) & np.uint32(0xFF)).astype(np.int64)

@@ -104,6 +104,12 @@ inline i32x16 mfma_i32_32x32x32_i8(u32x4 a, u32x4 b, i32x16 c) {
 }
 inline uint32_t mul_u24(uint32_t a, uint32_t b) { return (uint32_t)((uint64_t)(a & 0xffffffu) * (uint64_t)(b & 0xffffffu)); }
 
+inline uint32_t cvt_pk_u8_f32(float v, int sel, uint32_t old) {
+  const float r = nearbyintf(v);
+  const uint32_t b = r <= 0.f ? 0u : (r >= 255.f ? 255u : (uint32_t)r);
+  return (old & ~(0xffu << (8 * sel))) | (b << (8 * sel));
+}
+
 inline f32x16 mfma_32x32x2_f32(float a, float b, f32x16 c) {
   struct Ops { float a, b; } mine{a, b};
   EmuWave* w = emu_wave;

@@ -73,6 +73,11 @@ CASES = {
                             dict(ir=True, inp_res=1 / 127, bounds_up=[0, 64, 128], bounds_down=[0, 128, 256],
                                  out_bound=12.0, out_res=254.0, noise=0.04), "bf16", 2e-2),
     "bf16_interior_plain": (dict(T=80, D=128, E=3, F=128, k=2), dict(), "bf16", 2e-2),
+    # 256-column interior tiles: the 128 x 256 forward kernel (plain, clip + quantise, ADC without noise)
+    "bf16_wide_plain": (dict(T=90, D=256, E=3, F=256, k=2), dict(), "bf16", 2e-2),
+    "bf16_wide_ir_quant": (dict(T=90, D=256, E=3, F=256, k=2), dict(ir=True, inp_res=1 / 127, decay=0.01), "bf16", 2e-2),
+    "bf16_wide_adc": (dict(T=90, D=256, E=3, F=256, k=2),
+                      dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, bounds_up=[0, 96, 256]), "bf16", 2e-2),
     "f32_interior_ir_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(ir=True, decay=0.01), "f32", 1e-5),
     "f32_interior_quant_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(inp_res=1 / 127), "f32", 1e-5),
 }
@@ -210,7 +215,7 @@ def test_row_chunked_weight_gradient(emu_ops, dtype):
 
 
 @pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 128, 128, 60), (torch.bfloat16, 128, 128, 60),
-                                         (torch.bfloat16, 72, 40, 60)])
+                                         (torch.bfloat16, 72, 40, 60), (torch.bfloat16, 256, 256, 70)])
 def test_chained_projections(emu_ops, dtype, D, F, T):
     util.check_chained_projections(emu_ops, dtype=dtype, T=T, D=D, F=F)
 

@@ -273,8 +273,9 @@ def test_counter_noise_block_is_a_byte_matrix_product():
 
     def vec(key):
         out = []
-        for j, cj in enumerate((0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB, 0x165667, 0xD3A265, 0xFD7047, 0xB55A4F)):
-            w = ((key & 0xFFFFFF) * cj + key) & 0xFFFFFFFF
+        for j in range(8):
+            k = key ^ (0x5BD1E995 if j >= 4 else 0)
+            w = ((k & 0xFFFFFF) * (0x9E3779, 0x85EBCB, 0xC2B2AF, 0x27D4EB)[j % 4] + k) & 0xFFFFFFFF
             w ^= w >> 15
             for b in range(4):
                 v = (w >> (8 * b)) & 0xFF
