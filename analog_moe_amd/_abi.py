@@ -28,6 +28,7 @@ class FwdArgs(C.Structure):
         ("out_bound", C.c_float), ("out_res", C.c_float),
         ("relu", C.c_int32), ("range_flag", P),
         ("xq_out", P), ("ldxq", C.c_int64), ("xq_ir", P), ("xq_inp_res", C.c_float), ("x_is_quantized", C.c_int32),
+        ("code_out", P), ("ldcode", C.c_int64), ("code_scale_out", P),
     ]
 
 
@@ -77,6 +78,8 @@ PROTOTYPES = {
     "amoe_gate_reduce": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
     "amoe_ksum": (C.c_int, [I32, P, P, I64, I32, I32, P]),
     "amoe_gate_grad": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
+    "amoe_gate_reduce_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),
+    "amoe_gate_grad_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),
     "amoe_row_abs_max": (C.c_int, [I32, P, I64, I64, I32, P, P]),
     "amoe_weight_abs_max": (C.c_int, [I32, P, I32, I32, I32, I32, P, P]),
     "amoe_segment_sum": (C.c_int, [P, P, I32, I32, P, P]),
@@ -111,9 +114,14 @@ def set_bounds(args, bounds) -> None:
 
 
 class AmoeError(RuntimeError):
-    pass
+    rc = 0
+
+
+AMOE_EUNSUPPORTED = -6
 
 
 def check(lib, rc: int, what: str) -> None:
     if rc != 0:
-        raise AmoeError(f"{what}: {lib.amoe_strerror(rc).decode()} (rc={rc})")
+        err = AmoeError(f"{what}: {lib.amoe_strerror(rc).decode()} (rc={rc})")
+        err.rc = rc
+        raise err

@@ -5,6 +5,7 @@
 
 #include "gemm_rows.h"
 #include "gemm_fwd256.h"
+#include "gemm_bwdx256.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
 #include "weight_kernels.h"
@@ -99,10 +100,34 @@ int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
 
 // The 128 x 256 forward kernel for the usual training shapes (bf16, every tile interior, per-expert input
 // ranges, one max |W| per expert).  AMOE_EUNSUPPORTED: this launch is not one of them; the general kernel runs.
-template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2>
+template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
 int launch_fwd256_as(const RowsParams& p, int grid, hipStream_t st) {
-  auto k = &fwd256_kernel<A_MODE, ANALOG, NOISE, SPLIT2>;
+  auto k = &fwd256_kernel<A_MODE, ANALOG, NOISE, SPLIT2, ZCODES>;
   hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
+  return launch_rc();
+}
+
+// The 128 x 256 input-gradient kernel, for the same launches (and column tiles that are multiples of 256).  The
+// partial sums of the input-range gradient then cover 256 columns each; *n_count_blocks is the grid that ran.
+int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks) {
+  if (!rows_all_interior(p, MODE_BWDX, kFBK)) return AMOE_EUNSUPPORTED;
+  if (a->ir != nullptr && !a->ir_by_expert) return AMOE_EUNSUPPORTED;
+  if (a->x != nullptr && (!aligned(a->x, 16) || a->ldx % 8)) return AMOE_EUNSUPPORTED;   // 16-byte pieces of x rows
+  for (int t = 0; t < a->n_tiles; t++)
+    if ((a->tile_bounds[t + 1] - a->tile_bounds[t]) % kFCols) return AMOE_EUNSUPPORTED;
+  p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles, kFCols);
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
+  *n_count_blocks = grid;
+  const bool relu = a->relu_mask != 0, xc = a->xc_out != nullptr;
+  if (a->x == nullptr) {
+    hipLaunchKernelGGL((&bwdx256_kernel<false, false, false>), dim3(grid), dim3(kThreads), 0, st, p);
+  } else if (!relu) {
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, false, true>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<true, false, false>), dim3(grid), dim3(kThreads), 0, st, p);
+  } else {
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, true, true>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<true, true, false>), dim3(grid), dim3(kThreads), 0, st, p);
+  }
   return launch_rc();
 }
 
@@ -117,10 +142,22 @@ int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st
   if (a->n_tiles == 2 && !(analog && !a->x_is_quantized)) return AMOE_EUNSUPPORTED;
   p.n_col_blocks = a->N / kFCols;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
+  if (a->code_out && !analog) return AMOE_EUNSUPPORTED;
   if (!dac) return launch_fwd256_as<FA_PLAIN, false, false, false>(p, grid, st);
   if (!analog)
     return a->x_is_quantized ? launch_fwd256_as<FA_CODES, false, false, false>(p, grid, st)
                              : launch_fwd256_as<FA_DAC, false, false, false>(p, grid, st);
+  if (a->code_out) {
+    // codes leave instead of values: one output quantiser whose half range fits a byte, no second output
+    const float half = 0.5f * fmaxf(a->out_res, 1.0f / a->out_res);
+    if (a->n_tiles != 1 || a->xq_out || a->relu || !(half <= 127.f) || !aligned(a->code_out, 16) || a->ldcode % 16)
+      return AMOE_EUNSUPPORTED;
+    if (a->x_is_quantized)
+      return noisy ? launch_fwd256_as<FA_CODES, true, true, false, true>(p, grid, st)
+                   : launch_fwd256_as<FA_CODES, true, false, false, true>(p, grid, st);
+    return noisy ? launch_fwd256_as<FA_DAC, true, true, false, true>(p, grid, st)
+                 : launch_fwd256_as<FA_DAC, true, false, false, true>(p, grid, st);
+  }
   if (a->x_is_quantized)
     return noisy ? launch_fwd256_as<FA_CODES, true, true, false>(p, grid, st)
                  : launch_fwd256_as<FA_CODES, true, false, false>(p, grid, st);
@@ -256,9 +293,10 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
   if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->n_in_rows < 0 || a->n_out_rows < 0) return AMOE_EINVAL;
   if (a->M == 0) return AMOE_OK;
-  if (!a->x || !a->w || !a->out || !a->offsets || !a->in_index) return AMOE_ENULL;
+  if (!a->x || !a->w || (!a->out && !a->code_out) || !a->offsets || !a->in_index) return AMOE_ENULL;
+  if (a->code_out && (!a->code_scale_out || a->ldcode < a->N)) return AMOE_EINVAL;
   if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->K)) return rc;
-  if (a->ldx < a->K || a->ldo < a->N) return AMOE_ESHAPE;
+  if (a->ldx < a->K || (a->out && a->ldo < a->N)) return AMOE_ESHAPE;
   if (a->w_stride_n != 1 && a->w_stride_k != 1) return AMOE_EUNSUPPORTED;
   const bool gen_noise = a->noise == nullptr && a->noise_std > 0.f;
   const bool adc = a->out_bound > 0.f;
@@ -297,6 +335,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   p.xq_vec = a->xq_out && aligned(a->xq_out, 16) && (a->ldxq % 4 == 0);
   p.xq_stage = a->xq_out && aligned(a->xq_out, 16) && (a->ldxq % CH == 0);
   p.a_prequant = a->x_is_quantized;
+  p.code_out = a->code_out; p.ldcode = a->ldcode; p.code_scale_out = a->code_scale_out;
   const bool w_kc = a->w_stride_n != 1;
   p.a_vec = aligned(a->x, 16) && (a->ldx % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   p.w_vec = aligned(a->w, 16) && (a->w_stride_e % CH == 0) &&
@@ -315,6 +354,7 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
     const int rc = launch_fwd256(p, mode, a, st);
     if (rc != AMOE_EUNSUPPORTED) return rc;
   }
+  if (a->code_out) return AMOE_EUNSUPPORTED;      // only the kernel above writes codes
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (a->dtype == AMOE_F32)
     return w_kc ? launch_rows<float, true>(p, mode, grid, st) : launch_rows<float, false>(p, mode, grid, st);
@@ -477,14 +517,21 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.out_stage = aligned(a->grad_x_full, 16) && (a->ldo % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   p.xf_vec = a->x && aligned(a->x, 16) && (a->ldx % 4 == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, 4);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
-                                : launch_rows<uint16_t, true>(p, MODE_BWDX, grid, st);
+  int block_cols = kTileCols, n_count_blocks = grid;
+  int rc = AMOE_EUNSUPPORTED;
+  if (a->dtype == AMOE_BF16) {
+    rc = launch_bwdx256(p, a, st, &n_count_blocks);
+    if (rc == AMOE_OK) block_cols = kFCols;
+  }
+  if (rc == AMOE_EUNSUPPORTED)
+    rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
+                              : launch_rows<uint16_t, true>(p, MODE_BWDX, grid, st);
   if (rc) return rc;
   if (use_ir) {
     IrFinalizeParams f{};
-    f.M = a->M; f.n_tiles = a->n_tiles; f.KD_total = a->K;
+    f.M = a->M; f.n_tiles = a->n_tiles; f.KD_total = a->K; f.block_cols = block_cols;
     for (int t = 0; t <= a->n_tiles; t++) f.col_bounds[t] = a->tile_bounds[t];
-    f.irg_partial = p.irg_partial; f.notclip_count = p.notclip_count; f.n_blocks = grid;
+    f.irg_partial = p.irg_partial; f.notclip_count = p.notclip_count; f.n_blocks = n_count_blocks;
     f.ir = a->ir; f.ir_by_expert = a->ir_by_expert; f.offsets = a->offsets; f.E = a->E; f.ir_grad = a->ir_grad;
     f.relative = a->gradient_relative; f.scale = a->gradient_scale; f.decay = a->decay;
     f.min_pct = a->input_min_percentage;
@@ -552,6 +599,57 @@ int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate
     auto kf = &gate_grad_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
                        static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), (long long)T, (int)k, (int)D, vec);
+  }
+  return launch_rc();
+}
+
+static int codes_args_ok(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel, int32_t sel_is_i64,
+                         const void* a, const void* b, int64_t T, int32_t k, int32_t D) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
+  if (D % 16) return AMOE_EUNSUPPORTED;
+  if (T == 0) return AMOE_OK;
+  if (!codes || !scale || !sel || !a || !b) return AMOE_ENULL;
+  if (!aligned(codes, 16) || !aligned(scale, 4) || !aligned(sel, sel_is_i64 ? 8 : 4) || !aligned(a, esize(dtype)) ||
+      !aligned(b, 16))
+    return AMOE_EALIGN;
+  return AMOE_OK;
+}
+
+int amoe_gate_reduce_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel, int32_t sel_is_i64,
+                           const void* gate, void* y, int64_t T, int32_t k, int32_t D, void* stream) {
+  if (int rc = codes_args_ok(dtype, codes, scale, sel, sel_is_i64, gate, y, T, k, D)) return rc;
+  if (T == 0) return AMOE_OK;
+  const long long blocks = ((long long)T * (D / 16) + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &head_reduce_codes_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D);
+  } else {
+    auto kf = &head_reduce_codes_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D);
+  }
+  return launch_rc();
+}
+
+int amoe_gate_grad_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel, int32_t sel_is_i64,
+                         const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D, void* stream) {
+  if (int rc = codes_args_ok(dtype, codes, scale, sel, sel_is_i64, grad_gate, dy, T, k, D)) return rc;
+  if (T == 0) return AMOE_OK;
+  const long long blocks = ((long long)T + 4 * kCodeTokens - 1) / (4 * kCodeTokens);
+  if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == AMOE_F32) {
+    auto kf = &gate_grad_codes_kernel<float>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const float*>(dy), static_cast<float*>(grad_gate), (long long)T, (int)k, (int)D);
+  } else {
+    auto kf = &gate_grad_codes_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), (long long)T, (int)k, (int)D);
   }
   return launch_rc();
 }

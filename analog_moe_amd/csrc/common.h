@@ -240,21 +240,21 @@ __device__ __forceinline__ void find_row_tile(const int32_t* __restrict__ offset
   __syncthreads();
 }
 
-// Feature blocks of kTileCols columns that restart at every K-tile bound, so that one block
+// Feature blocks of `width` columns (kTileCols unless said otherwise) that restart at every K-tile bound, so that one block
 // lies inside one K-tile.  Block b -> (first column, end column, K-tile).
 struct ColBlock { int c0, c1, tile; };
-__device__ __host__ inline int count_col_blocks(const int32_t* bounds, int n_tiles) {
+__device__ __host__ inline int count_col_blocks(const int32_t* bounds, int n_tiles, int width = kTileCols) {
   int n = 0;
-  for (int t = 0; t < n_tiles; t++) n += (bounds[t + 1] - bounds[t] + kTileCols - 1) / kTileCols;
+  for (int t = 0; t < n_tiles; t++) n += (bounds[t + 1] - bounds[t] + width - 1) / width;
   return n;
 }
-__device__ __forceinline__ ColBlock find_col_block(const int32_t* bounds, int n_tiles, int b) {
+__device__ __forceinline__ ColBlock find_col_block(const int32_t* bounds, int n_tiles, int b, int width = kTileCols) {
   ColBlock r{0, 0, 0};
   for (int t = 0; t < n_tiles; t++) {
-    int nb = (bounds[t + 1] - bounds[t] + kTileCols - 1) / kTileCols;
+    int nb = (bounds[t + 1] - bounds[t] + width - 1) / width;
     if (b < nb) {
-      r.c0 = bounds[t] + b * kTileCols;
-      r.c1 = (r.c0 + kTileCols < bounds[t + 1]) ? r.c0 + kTileCols : bounds[t + 1];
+      r.c0 = bounds[t] + b * width;
+      r.c1 = (r.c0 + width < bounds[t + 1]) ? r.c0 + width : bounds[t + 1];
       r.tile = t;
       return r;
     }

@@ -26,8 +26,9 @@ enum { FA_PLAIN = 0, FA_DAC = 1, FA_CODES = 2 };   // what the gathered operand 
 
 // A_MODE: see above.  ANALOG: ADC with rounding + rescale by the input range, after the generated noise if NOISE;
 // otherwise the accumulator leaves as it is (times inp_res * ir for code operands).  SPLIT2: exactly two K-tiles
-// (needs ANALOG).
-template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2>
+// (needs ANALOG).  ZCODES: the result leaves as its ADC codes + 128, one byte each (and the expert's step and input
+// range go to code_scale_out), instead of as values.
+template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
 __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p) {
   using T = uint16_t;
   constexpr int BK = kFBK, CH = 8;
@@ -39,6 +40,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
   constexpr int OUT_ROWS = 64;                      // rows per output pass
   static_assert(OUT_ROWS * LDO <= 2 * STAGE, "output staging must fit the stage buffers");
   static_assert((!SPLIT2 || ANALOG) && (!NOISE || ANALOG), "the packed first tile holds ADC codes");
+  static_assert(!ZCODES || (ANALOG && !SPLIT2), "a result leaves as ADC codes only after a single output quantiser");
   constexpr bool CODES = A_MODE != FA_PLAIN;        // the matrix unit sees integer codes: scale the accumulator
 
   __shared__ __attribute__((aligned(16))) T sStage[2 * STAGE];
@@ -276,6 +278,8 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
                     const float first = (float)((packed[fi][ti][q] >> (8 * j)) & 0xffu) - 128.0f;
                     acc[fi][ti][4 * q + j] = (first * u_qinv) * ir_first + (code * u_qinv) * ir_t;
                   }
+                } else if constexpr (ZCODES) {
+                  word = cvt_pk_u8_f32(code + 128.0f, j, word);
                 } else {
                   acc[fi][ti][4 * q + j] = (code * u_qinv) * ir_t;
                 }
@@ -283,10 +287,20 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
               if constexpr (SPLIT2) {
                 if (t == 0) packed[fi][ti][q] = word;
               }
+              if constexpr (ZCODES) {     // straight to the staged tile (the stage buffers are idle by now)
+                *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(sStage) + rl * (kFCols + 16) + wc * 128 +
+                                             fi * 32 + 8 * q + 4 * lh) = word;
+              }
             }
           }
         }
         if (SPLIT2 && t == 0) ir_first = ir_t;
+        if constexpr (ZCODES) {
+          if (tid == 0 && cb == 0 && row0 == p.offsets[e]) {     // once per expert that has rows
+            p.code_scale_out[2 * e] = u_qinv;
+            p.code_scale_out[2 * e + 1] = ir_t;
+          }
+        }
       } else if constexpr (CODES) {
         const float s1 = p.inp_res;
 #pragma unroll
@@ -298,6 +312,30 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
       }
     }
 
+    if constexpr (ZCODES) {
+      // one byte per result: rows of 256 bytes (+ 16) through LDS, whole 256-byte row segments out
+      constexpr int LDC = kFCols + 16;
+      const uint8_t* __restrict__ sC = reinterpret_cast<const uint8_t*>(sStage);   // filled by the output stage
+      __syncthreads();
+      constexpr int CPRC = kFCols / 16;            // 16 chunks of 16 bytes per row
+      constexpr int RPPC = kThreads / CPRC;        // 16 rows per pass
+#pragma unroll
+      for (int i0 = 0; i0 < kTileRows / RPPC; i0 += 4) {
+        Raw seg[4];
+        int orow[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int rl = tid / CPRC + RPPC * (i0 + i);
+          orow[i] = sOrow[rl];
+          seg[i] = *reinterpret_cast<const Raw*>(&sC[rl * LDC + (tid % CPRC) * 16]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (orow[i] >= 0) store_streaming(p.code_out + (int64_t)orow[i] * p.ldcode + c0 + (tid % CPRC) * 16, seg[i]);
+      }
+      __syncthreads();
+      continue;
+    }
     if (p.relu) {
 #pragma unroll
       for (int fi = 0; fi < 4; fi++)

@@ -61,6 +61,7 @@ struct RowsParams {
   int32_t* range_flag;
   void* xq_out; int64_t ldxq; const float* xq_ir; float xq_inp_res; int xq_stage, xq_vec;  // DAC image of the result
   int a_prequant;                    // the gathered operand already is such an image: no input stage
+  uint8_t* code_out; int64_t ldcode; float* code_scale_out;   // the result as ADC codes + 128 (gemm_fwd256.h)
   // input gradient
   const void* xf; int64_t ldxf; const int32_t* xf_index; const void* gate;
   float* irg_partial; int32_t* notclip_count; int relu_mask;
@@ -880,6 +881,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 // Sum the column-block partials into ir_grad[M, n_tiles] and apply the scaling and decay rules.
 struct IrFinalizeParams {
   int M, n_tiles, KD_total;      // KD_total = columns of x (for the un-clipped fraction)
+  int block_cols;                // width of the column blocks the partial sums were made over
   int col_bounds[kMaxTiles + 1];
   const float* irg_partial; const int32_t* notclip_count; int n_blocks;
   const float* ir; int ir_by_expert; const int32_t* offsets; int E; float* ir_grad;
@@ -914,7 +916,7 @@ __global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFina
   }
   int cb = 0;
   for (int t = 0; t < p.n_tiles; t++) {
-    const int nb = (p.col_bounds[t + 1] - p.col_bounds[t] + kTileCols - 1) / kTileCols;
+    const int nb = (p.col_bounds[t + 1] - p.col_bounds[t] + p.block_cols - 1) / p.block_cols;
     float s = 0.f;
     for (int b = 0; b < nb; b++) s += p.irg_partial[(int64_t)(cb + b) * p.M + r];
     cb += nb;

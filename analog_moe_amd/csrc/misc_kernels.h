@@ -79,6 +79,144 @@ __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict
   }
 }
 
+// ---- the same two companions for a k-head tensor stored as ADC codes -----------------------------------------
+// z[r, d] = ((code[r, d] - 128) * scale[e][0]) * scale[e][1], e = sel[r] (the expert of flat row r = t*k + j).
+__device__ __forceinline__ int code_row_expert(const void* sel, int sel_is_i64, long long r) {
+  return sel_is_i64 ? (int)static_cast<const long long*>(sel)[r] : static_cast<const int32_t*>(sel)[r];
+}
+__device__ __forceinline__ void codes_unpack16(const Raw& r, float a, float b, float (&v)[16]) {
+#pragma unroll
+  for (int w = 0; w < 4; w++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[4 * w + i] = (((float)((r[w] >> (8 * i)) & 0xffu) - 128.0f) * a) * b;
+}
+
+// One thread per (token, 16 codes): y[t, d] = sum_j gate[t*k+j] * z[t*k+j, d], fp32, ascending j.  D % 16 == 0.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void head_reduce_codes_kernel(const uint8_t* __restrict__ codes,
+                                                                      const float* __restrict__ scale,
+                                                                      const void* __restrict__ sel, int sel_is_i64,
+                                                                      const T* __restrict__ gate, T* __restrict__ y,
+                                                                      long long rows, int k, int D) {
+  const int chunks = D / 16;
+  const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+  if (idx >= rows * chunks) return;
+  const long long t = idx / chunks;
+  const int d = (int)(idx % chunks) * 16;
+  float acc[16];
+#pragma unroll
+  for (int q = 0; q < 16; q++) acc[q] = 0.f;
+  for (int j = 0; j < k; j++) {
+    const long long r = t * k + j;
+    const Raw c = __builtin_nontemporal_load(reinterpret_cast<const Raw*>(codes + r * (long long)D + d));
+    const int e = code_row_expert(sel, sel_is_i64, r);
+    float v[16];
+    codes_unpack16(c, scale[2 * e], scale[2 * e + 1], v);
+    const float gt = Elem<T>::load(gate + r);
+#pragma unroll
+    for (int q = 0; q < 16; q++) acc[q] += gt * v[q];
+  }
+  T* out = y + t * (long long)D + d;
+  if constexpr (sizeof(T) == 2) {
+    float lo[8], hi[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) { lo[q] = acc[q]; hi[q] = acc[8 + q]; }
+    store_streaming(out, raw_pack<T>(lo));
+    store_streaming(out + 8, raw_pack<T>(hi));
+  } else {
+#pragma unroll
+    for (int q = 0; q < 16; q += 4) {
+      float f[4] = {acc[q], acc[q + 1], acc[q + 2], acc[q + 3]};
+      store_streaming(out + q, raw_pack<T>(f));
+    }
+  }
+}
+
+// grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>.  A wave takes kCodeTokens tokens at once (their loads are all in
+// flight together); a lane owns runs of 16 columns.  sum (c - 128) * dy = sum c * dy - 128 * sum dy: the products
+// run on the bytes as they are, the row's two scale factors multiply the finished sum.  D % 16 == 0.
+constexpr int kCodeTokens = 2;
+template <typename T>
+__global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t* __restrict__ codes,
+                                                                    const float* __restrict__ scale,
+                                                                    const void* __restrict__ sel, int sel_is_i64,
+                                                                    const T* __restrict__ dy, T* __restrict__ out,
+                                                                    long long tokens, int k, int D) {
+  constexpr int JB = 8, TK = kCodeTokens;
+  const int lane = threadIdx.x & 63;
+  const long long t0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * TK;
+  if (t0 >= tokens) return;
+  for (int j0 = 0; j0 < k; j0 += JB) {
+    float s[TK][JB], sb[TK];
+#pragma unroll
+    for (int u = 0; u < TK; u++) {
+      sb[u] = 0.f;
+#pragma unroll
+      for (int jj = 0; jj < JB; jj++) s[u][jj] = 0.f;
+    }
+    for (int d = lane * 16; d < D; d += 64 * 16) {
+      Raw rc[TK][JB], rd[TK][sizeof(T) == 2 ? 2 : 4];
+#pragma unroll
+      for (int u = 0; u < TK; u++) {
+        const long long t = t0 + u < tokens ? t0 + u : t0;        // a wave past the end repeats its first token
+#pragma unroll
+        for (int jj = 0; jj < JB; jj++)
+          rc[u][jj] = j0 + jj < k ? __builtin_nontemporal_load(reinterpret_cast<const Raw*>(codes + (t * k + j0 + jj) * (long long)D + d))
+                                  : raw_zero();
+#pragma unroll
+        for (int q = 0; q < (sizeof(T) == 2 ? 2 : 4); q++)
+          rd[u][q] = *reinterpret_cast<const Raw*>(dy + t * (long long)D + d + q * (16 / (int)sizeof(T)));
+      }
+#pragma unroll
+      for (int u = 0; u < TK; u++) {
+        float b[16];
+        if constexpr (sizeof(T) == 2) {
+          float lo[8], hi[8];
+          raw_unpack<T>(rd[u][0], lo);
+          raw_unpack<T>(rd[u][1], hi);
+#pragma unroll
+          for (int q = 0; q < 8; q++) { b[q] = lo[q]; b[8 + q] = hi[q]; }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) b[4 * q + i] = as_f32(rd[u][q][i]);
+        }
+        float bs = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; q++) bs += b[q];
+        sb[u] += bs;
+#pragma unroll
+        for (int jj = 0; jj < JB; jj++) {
+          float acc = 0.f;
+#pragma unroll
+          for (int w = 0; w < 4; w++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc += (float)((rc[u][jj][w] >> (8 * i)) & 0xffu) * b[4 * w + i];
+          s[u][jj] += acc;
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < TK; u++) {
+      float vb = sb[u];
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) vb += wave_shfl_xor(vb, d);
+#pragma unroll
+      for (int jj = 0; jj < JB; jj++) {
+        float v = s[u][jj];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) v += wave_shfl_xor(v, d);
+        if (lane == 0 && j0 + jj < k && t0 + u < tokens) {
+          const long long r = (t0 + u) * k + j0 + jj;
+          const int e = code_row_expert(sel, sel_is_i64, r);
+          out[r] = Elem<T>::cvt(((v - 128.0f * vb) * scale[2 * e]) * scale[2 * e + 1]);
+        }
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void row_abs_max_kernel(const T* __restrict__ x, long long ldx, long long rows,
                                                                 int K, float* __restrict__ out) {

@@ -71,8 +71,9 @@ def ir_tables(input_range: Optional[torch.Tensor], E: int, cfg: FFNConfig):
 
 
 def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
-    """Sort, both projections and the gate reduction.  Returns (y, p1, z, perm, in_index, offsets, ir_up,
-    ir_dn): the result and what the backward pass reads again."""
+    """Sort, both projections and the gate reduction.  Returns (y, p1, z, perm, in_index, offsets, z_scale, ir_up,
+    ir_dn): the result and what the backward pass reads again.  z is the down-projection's k-head result
+    [T*k, D], either as values (z_scale empty) or as uint8 ADC codes with z_scale [E, 2] (``ops.dequant_codes``)."""
     T, D = x.shape
     E, _, F = keys.shape
     k = sel_idx.shape[-1]
@@ -105,15 +106,29 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
                       noise_seed_dev=cfg.noise_seed_dev, xq_ir=ir_dn[:, 0].contiguous() if chain else None,
                       xq_inp_res=cfg.inp_res, **common)
     p1, p1q = p1 if chain else (p1, None)
-    z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, ir=ir_dn,
-                     bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
-                     noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
-    y = ops.gate_reduce(z, gate)
-    return y, p1, z, perm, in_index, offsets, ir_up, ir_dn
+    down = dict(ir=ir_dn, bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
+                noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
+    if chain and z_as_codes(p1q, values, cfg):
+        # the down-projection's result is read twice more and never as a matrix operand (gate reduction now, gate
+        # gradient in the backward pass): it is kept as its ADC codes, one byte per value, with two factors per expert
+        z, z_scale = ops.cvmm_fwd(p1q, values, sel_sorted, offsets, perm, None, M, want_codes=True, **down)
+        y = ops.gate_reduce_codes(z, z_scale, sel_idx, gate)
+    else:
+        z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, **down)
+        z_scale = torch.empty(0, dtype=torch.float32, device=x.device)
+        y = ops.gate_reduce(z, gate)
+    return y, p1, z, perm, in_index, offsets, z_scale, ir_up, ir_dn
 
 
-def ffn_backward(dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn, cfg: FFNConfig,
-                 want_ir_grad: bool):
+def z_as_codes(p1q: torch.Tensor, values: torch.Tensor, cfg: FFNConfig) -> bool:
+    """Whether the down-projection leaves its result as ADC codes (a pure function of shapes and settings)."""
+    return ops.codes_supported(p1q, values, ir_by_expert=True, inp_res=cfg.inp_res, n_tiles=_n_tiles(cfg.bounds_down),
+                               out_bound=cfg.out_bound, out_res=cfg.out_res, noise=cfg.noise_down,
+                               per_channel=cfg.noise_per_channel)
+
+
+def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn,
+                 cfg: FFNConfig, want_ir_grad: bool):
     """Returns (grad_x, grad_keys, grad_values, grad_ir [2, E, n_tiles] fp32 or None, grad_gate)."""
     E = keys.shape[0]
     k = gate.shape[-1]
@@ -136,7 +151,10 @@ def ffn_backward(dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_u
     main, side = torch.cuda.current_stream(), _side_stream(x.device)
     side.wait_stream(main)
     with torch.cuda.stream(side):
-        grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
+        if z.dtype == torch.uint8:
+            grad_gate = ops.gate_grad_codes(z, z_scale, sel_idx, dy, k).view(gate.shape)
+        else:
+            grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
         grad_x = ops.ksum(full, k) if k > 1 else full
     grad_gate.record_stream(main)
     grad_x.record_stream(main)
@@ -158,9 +176,9 @@ class AnalogMoEFFN(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
-        y, p1, z, perm, in_index, offsets, ir_up, ir_dn = ffn_forward(x, keys, values, input_range, gate,
-                                                                      sel_idx, cfg)
-        ctx.save_for_backward(x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn)
+        y, p1, z, perm, in_index, offsets, z_scale, ir_up, ir_dn = ffn_forward(x, keys, values, input_range, gate,
+                                                                               sel_idx, cfg)
+        ctx.save_for_backward(x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn)
         ctx.cfg = cfg
         ctx.ir_shape = None if input_range is None else input_range.shape
         ctx.ir_dtype = None if input_range is None else input_range.dtype
@@ -168,9 +186,9 @@ class AnalogMoEFFN(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
-        x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn = ctx.saved_tensors
+        x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn = ctx.saved_tensors
         grad_x, grad_keys, grad_values, grad_ir, grad_gate = ffn_backward(
-            dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn, ctx.cfg,
+            dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn, ctx.cfg,
             ctx.needs_input_grad[3])
         if grad_ir is not None:
             grad_ir = grad_ir.reshape(ctx.ir_shape).to(ctx.ir_dtype)

@@ -289,10 +289,10 @@ def _cfg(values) -> ffn.FFNConfig:
 @torch.library.custom_op(
     "amoe::ffn_fwd", mutates_args=(),
     schema="(Tensor x, Tensor keys, Tensor values, Tensor? input_range, Tensor gate, Tensor sel_idx, "
-           + _CFG_SCHEMA + ") -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
+           + _CFG_SCHEMA + ") -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)")
 def ffn_fwd(x, keys, values, input_range, gate, sel_idx, *cfg):
-    """(y, p1, z, perm, in_index, offsets): the result and what ``amoe::ffn_bwd`` reads again."""
-    return ffn.ffn_forward(x, keys, values, input_range, gate, sel_idx, _cfg(cfg))[:6]
+    """(y, p1, z, perm, in_index, offsets, z_scale): the result and what ``amoe::ffn_bwd`` reads again."""
+    return ffn.ffn_forward(x, keys, values, input_range, gate, sel_idx, _cfg(cfg))[:7]
 
 
 @ffn_fwd.register_fake
@@ -300,21 +300,29 @@ def _(x, keys, values, input_range, gate, sel_idx, *cfg):
     T, k = x.shape[0], sel_idx.shape[-1]
     M = T * k
     i32 = dict(dtype=torch.int32, device=x.device)
-    return (x.new_empty((T, values.shape[2])), x.new_empty((M, keys.shape[2])), x.new_empty((M, values.shape[2])),
-            torch.empty(M, **i32), torch.empty(M, **i32), torch.empty(keys.shape[0] + 1, **i32))
+    c = _cfg(cfg)
+    E, F, D = values.shape
+    # (the same decision ffn_forward makes: a function of shapes and settings only)
+    chain = input_range is not None and c.inp_res > 0 and (c.bounds_down is None or len(c.bounds_down) == 2)
+    codes = chain and ffn.z_as_codes(x.new_empty((M, F)), values, c)
+    z = torch.empty((M, D), dtype=torch.uint8, device=x.device) if codes else x.new_empty((M, D))
+    z_scale = torch.empty((E, 2) if codes else (0,), dtype=torch.float32, device=x.device)
+    return (x.new_empty((T, D)), x.new_empty((M, keys.shape[2])), z,
+            torch.empty(M, **i32), torch.empty(M, **i32), torch.empty(E + 1, **i32), z_scale)
 
 
 @torch.library.custom_op(
     "amoe::ffn_bwd", mutates_args=(),
-    schema="(Tensor dy, Tensor x, Tensor keys, Tensor values, Tensor? input_range, Tensor gate, Tensor p1, "
-           "Tensor z, Tensor perm, Tensor in_index, Tensor offsets, bool want_ir_grad, " + _CFG_SCHEMA
-           + ") -> (Tensor, Tensor, Tensor, Tensor, Tensor)")
-def ffn_bwd(dy, x, keys, values, input_range, gate, p1, z, perm, in_index, offsets, want_ir_grad, *cfg):
+    schema="(Tensor dy, Tensor x, Tensor keys, Tensor values, Tensor? input_range, Tensor gate, Tensor sel_idx, "
+           "Tensor p1, Tensor z, Tensor z_scale, Tensor perm, Tensor in_index, Tensor offsets, bool want_ir_grad, "
+           + _CFG_SCHEMA + ") -> (Tensor, Tensor, Tensor, Tensor, Tensor)")
+def ffn_bwd(dy, x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, want_ir_grad,
+            *cfg):
     """(grad_x, grad_keys, grad_values, grad_input_range or empty, grad_gate)."""
     c = _cfg(cfg)
     ir_up, ir_dn = ffn.ir_tables(input_range, keys.shape[0], c)
-    gx, gk, gv, gir, gg = ffn.ffn_backward(dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn,
-                                           c, want_ir_grad)
+    gx, gk, gv, gir, gg = ffn.ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets,
+                                           ir_up, ir_dn, c, want_ir_grad)
     if gir is None:
         gir = torch.empty(_EMPTY_SHAPE, dtype=torch.float32, device=x.device)
     else:
@@ -323,7 +331,7 @@ def ffn_bwd(dy, x, keys, values, input_range, gate, p1, z, perm, in_index, offse
 
 
 @ffn_bwd.register_fake
-def _(dy, x, keys, values, input_range, gate, p1, z, perm, in_index, offsets, want_ir_grad, *cfg):
+def _(dy, x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, want_ir_grad, *cfg):
     if input_range is not None and want_ir_grad:
         gir = torch.empty_like(input_range)
     else:
@@ -333,19 +341,19 @@ def _(dy, x, keys, values, input_range, gate, p1, z, perm, in_index, offsets, wa
 
 def _ffn_setup_context(ctx, inputs, output):
     x, keys, values, input_range, gate, sel_idx = inputs[:6]
-    _, p1, z, perm, in_index, offsets = output
-    ctx.save_for_backward(x, keys, values, input_range, gate, p1, z, perm, in_index, offsets)
+    _, p1, z, perm, in_index, offsets, z_scale = output
+    ctx.save_for_backward(x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets)
     ctx.cfg = tuple(inputs[6:])
     ctx.want_ir_grad = input_range is not None and ctx.needs_input_grad[3]
     ctx.set_materialize_grads(False)
 
 
 def _ffn_autograd(ctx, dy, *_unused):
-    x, keys, values, input_range, gate, p1, z, perm, in_index, offsets = ctx.saved_tensors
+    x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets = ctx.saved_tensors
     if dy is None:
         return (None,) * (6 + _N_CFG)
-    gx, gk, gv, gir, gg = torch.ops.amoe.ffn_bwd(dy, x, keys, values, input_range, gate, p1, z, perm, in_index,
-                                                 offsets, ctx.want_ir_grad, *ctx.cfg)
+    gx, gk, gv, gir, gg = torch.ops.amoe.ffn_bwd(dy, x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, perm,
+                                                 in_index, offsets, ctx.want_ir_grad, *ctx.cfg)
     return (gx, gk, gv, gir if ctx.want_ir_grad else None, gg, None) + (None,) * _N_CFG
 
 

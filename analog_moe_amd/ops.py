@@ -96,22 +96,51 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
              noise_std: float = 0.0, noise_seed: int = 0, wmax: Optional[torch.Tensor] = None,
              out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
              ir_by_expert: bool = False, noise_seed_dev: Optional[torch.Tensor] = None,
-             xq_ir: Optional[torch.Tensor] = None, xq_inp_res: float = -1.0, x_is_quantized: bool = False):
+             xq_ir: Optional[torch.Tensor] = None, xq_inp_res: float = -1.0, x_is_quantized: bool = False,
+             want_codes: bool = False):
     """out[out_index[i]] = analog(x[in_index[i]]) @ w[sel_sorted[i]] -> [n_out_rows, N].
     ir: [M, n_tiles] per sorted position, or the [E, n_tiles] table with ir_by_expert.
     noise_seed_dev: optional int64 device word added to noise_seed by the kernel.
     xq_ir ([E] fp32) + xq_inp_res: also return the input-stage image of the result for the projection
-    that follows (-> (out, xq)); x_is_quantized: x is such an image made for this call."""
+    that follows (-> (out, xq)); x_is_quantized: x is such an image made for this call.
+    want_codes: return the result as its ADC codes instead -> (codes uint8 [n_out_rows, N] = code + 128,
+    scale fp32 [E, 2]) with result = ((code - 128) * scale[e, 0]) * scale[e, 1]; raises AmoeError (rc
+    AMOE_EUNSUPPORTED) where the library has no such kernel for the call (see ``codes_supported``)."""
     _need_gpu(x, w, sel_sorted, offsets, in_index, out_index, ir, abs_max, noise, wmax)
     x2 = _rows2d(x)
     if w.stride(2) != 1 and w.stride(1) != 1:
         w = w.contiguous()
+    if want_codes:
+        codes = torch.empty((n_out_rows, w.shape[2]), dtype=torch.uint8, device=x2.device)
+        scale = torch.empty((w.shape[0], 2), dtype=torch.float32, device=x2.device)
+        dummy = torch.empty((0, w.shape[2]), dtype=x2.dtype, device=x2.device)
+        raw.cvmm_fwd(get_lib(), _stream(x2), x2, w, dummy, sel_sorted, offsets, in_index, out_index, _f32c(ir),
+                     _f32c(abs_max), inp_res, bounds, _f32c(noise), noise_std, noise_seed, _f32c(wmax), out_bound,
+                     out_res, relu, None, ir_by_expert, noise_seed_dev, None, None, -1.0, x_is_quantized,
+                     code_out=codes, code_scale_out=scale)
+        return codes, scale
     out = torch.empty((n_out_rows, w.shape[2]), dtype=x2.dtype, device=x2.device)
     xq = torch.empty_like(out) if xq_ir is not None else None
     raw.cvmm_fwd(get_lib(), _stream(x2), x2, w, out, sel_sorted, offsets, in_index, out_index, _f32c(ir),
                  _f32c(abs_max), inp_res, bounds, _f32c(noise), noise_std, noise_seed, _f32c(wmax), out_bound,
                  out_res, relu, None, ir_by_expert, noise_seed_dev, xq, _f32c(xq_ir), xq_inp_res, x_is_quantized)
     return out if xq is None else (out, xq)
+
+
+def codes_supported(x: torch.Tensor, w: torch.Tensor, *, ir_by_expert: bool, inp_res: float, n_tiles: int,
+                    out_bound: float, out_res: float, noise: Optional[torch.Tensor], per_channel: bool) -> bool:
+    """Whether ``cvmm_fwd(..., want_codes=True)`` has a kernel for this call: the 128 x 256 forward kernel
+    with an output quantiser of at most 254 states (bf16, every tile interior: N a multiple of 256, K of 32,
+    16-byte aligned rows; per-expert input ranges with input quantisation; one max |W| per expert; no injected
+    noise; one K-tile).  A pure function of shapes and settings, so that traced code can rely on it."""
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not w.is_contiguous():
+        return False
+    E, K, N = w.shape
+    x2_stride = x.stride(-2) if x.dim() >= 2 else K
+    half = 0.5 * max(out_res, 1.0 / out_res) if out_res > 0 else 0.0
+    return (ir_by_expert and inp_res > 0 and n_tiles == 1 and out_bound > 0 and 0 < half <= 127 and noise is None
+            and not per_channel and N % 256 == 0 and K % 32 == 0 and x2_stride % 8 == 0 and x.stride(-1) == 1
+            and x.numel() * 2 < 2 ** 31 and (K * N) * 2 < 2 ** 31)
 
 
 def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,
@@ -173,6 +202,35 @@ def gate_reduce(z: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
     y = torch.empty((T, D), dtype=z2.dtype, device=z2.device)
     raw.gate_reduce(get_lib(), _stream(z2), z2, gate_c, y, T, k, D)
     return y
+
+
+def gate_reduce_codes(codes: torch.Tensor, scale: torch.Tensor, sel: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """``gate_reduce`` of a k-head tensor stored as ADC codes (``cvmm_fwd(..., want_codes=True)``); sel [..., k]: the
+    expert of every (token, head)."""
+    _need_gpu(codes, scale, sel, gate)
+    k = gate.shape[-1]
+    T, D = codes.shape[0] // k, codes.shape[1]
+    gate_c = gate.detach().reshape(-1).contiguous()
+    sel_c = sel.detach().reshape(-1).contiguous()
+    y = torch.empty((T, D), dtype=gate_c.dtype, device=codes.device)
+    raw.gate_reduce_codes(get_lib(), _stream(codes), codes, scale, sel_c, gate_c, y, T, k, D)
+    return y
+
+
+def gate_grad_codes(codes: torch.Tensor, scale: torch.Tensor, sel: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:
+    _need_gpu(codes, scale, sel, dy)
+    d2 = _rows2d(dy).contiguous()
+    T, D = d2.shape
+    sel_c = sel.detach().reshape(-1).contiguous()
+    out = torch.empty((T, k), dtype=d2.dtype, device=d2.device)
+    raw.gate_grad_codes(get_lib(), _stream(d2), codes, scale, sel_c, d2, out, T, k, D)
+    return out
+
+
+def dequant_codes(codes: torch.Tensor, scale: torch.Tensor, sel: torch.Tensor) -> torch.Tensor:
+    """The values behind a code tensor, fp32 (tests, debugging): ((code - 128) * scale[e, 0]) * scale[e, 1]."""
+    e = sel.reshape(-1).long()
+    return ((codes.float() - 128.0) * scale[e, 0:1]) * scale[e, 1:2]
 
 
 def ksum(full: torch.Tensor, k: int) -> torch.Tensor:

@@ -67,8 +67,10 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
              inp_res: float = -1.0, bounds: Optional[Sequence[int]] = None, noise=None, noise_std: float = 0.0,
              noise_seed: int = 0, wmax=None, out_bound: float = -1.0, out_res: float = -1.0, relu: bool = False,
              range_flag=None, ir_by_expert: bool = False, noise_seed_dev=None, xq_out=None, xq_ir=None,
-             xq_inp_res: float = -1.0, x_is_quantized: bool = False):
-    """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N]."""
+             xq_inp_res: float = -1.0, x_is_quantized: bool = False, code_out=None, code_scale_out=None):
+    """x [R_in, K]; w [E, K, N] (any strides with K or N contiguous); out [R_out, N] -- or, with code_out
+    (uint8 [R_out, N]) and code_scale_out (fp32 [E, 2]), the result as ADC codes and ``out`` a dummy of the
+    right shape that is not written."""
     _rows(x, "x"); _rows(out, "out")
     a = FwdArgs()
     a.dtype = dtype_code(x)
@@ -77,12 +79,19 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
     E, K, N = w.shape
     if x.shape[1] != K or out.shape[1] != N:
         raise ValueError("x / w / out shapes do not match")
+    if code_out is not None:
+        if code_out.dtype != torch.uint8 or code_out.dim() != 2 or code_out.shape[1] != N or not code_out.is_contiguous():
+            raise ValueError("code_out must be a contiguous uint8 tensor [rows, N]")
+        if code_scale_out is None or code_scale_out.dtype != torch.float32 or code_scale_out.numel() != 2 * E:
+            raise ValueError("code_scale_out must be fp32 [E, 2]")
+        a.code_out, a.ldcode, a.code_scale_out = _p(code_out), code_out.stride(0), _p(code_scale_out)
     M = in_index.numel()
     a.M, a.N, a.K, a.E = M, N, K, E
-    a.n_in_rows, a.n_out_rows = x.shape[0], out.shape[0]
+    n_out_rows = out.shape[0] if code_out is None else code_out.shape[0]
+    a.n_in_rows, a.n_out_rows = x.shape[0], n_out_rows
     a.x, a.ldx = _p(x), x.stride(0)
     a.w, a.w_stride_e, a.w_stride_k, a.w_stride_n = _p(w), w.stride(0), w.stride(1), w.stride(2)
-    a.out, a.ldo = _p(out), out.stride(0)
+    a.out, a.ldo = (None if code_out is not None and out.numel() == 0 else _p(out)), out.stride(0)
     a.sel_sorted, a.offsets = _p(_i32(sel_sorted, "sel_sorted")), _p(_i32(offsets, "offsets"))
     a.in_index, a.out_index = _p(_i32(in_index, "in_index")), _p(_i32(out_index, "out_index"))
     set_bounds(a, [0, K] if bounds is None else bounds)
@@ -92,9 +101,9 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
     a.ir, a.abs_max, a.inp_res = _p(_f32(ir, "ir")), _p(_f32(abs_max, "abs_max")), float(inp_res)
     if noise is not None:
         _f32(noise, "noise")
-        if noise.numel() != a.n_tiles * out.shape[0] * N:
+        if noise.numel() != a.n_tiles * n_out_rows * N:
             raise ValueError("noise must be [n_tiles, out rows, N]")
-        a.noise, a.noise_tile_stride, a.ldnoise = _p(noise), out.shape[0] * N, N
+        a.noise, a.noise_tile_stride, a.ldnoise = _p(noise), n_out_rows * N, N
     a.noise_std, a.noise_seed = float(noise_std), int(noise_seed) & 0xFFFFFFFFFFFFFFFF
     if noise_seed_dev is not None:
         if noise_seed_dev.dtype != torch.int64 or noise_seed_dev.numel() != 1:
@@ -107,7 +116,7 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
     a.relu, a.range_flag = int(bool(relu)), _p(range_flag)
     if xq_out is not None:
         _rows(xq_out, "xq_out")
-        if xq_out.dtype != x.dtype or xq_out.shape != out.shape:
+        if xq_out.dtype != x.dtype or tuple(xq_out.shape) != (n_out_rows, N):
             raise ValueError("xq_out must match out")
         a.xq_out, a.ldxq, a.xq_ir, a.xq_inp_res = _p(xq_out), xq_out.stride(0), _p(_f32(xq_ir, "xq_ir")), float(xq_inp_res)
     a.x_is_quantized = int(bool(x_is_quantized))
@@ -193,6 +202,16 @@ def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=No
 
 def gate_reduce(lib, stream, z, gate, y, T: int, k: int, D: int):
     check(lib, lib.amoe_gate_reduce(dtype_code(z), _p(z), _p(gate), _p(y), T, k, D, stream), "amoe_gate_reduce")
+
+
+def gate_reduce_codes(lib, stream, codes, scale, sel, gate, y, T: int, k: int, D: int):
+    check(lib, lib.amoe_gate_reduce_codes(dtype_code(y), _p(codes), _p(scale), _p(sel), int(sel.dtype == torch.int64),
+                                          _p(gate), _p(y), T, k, D, stream), "amoe_gate_reduce_codes")
+
+
+def gate_grad_codes(lib, stream, codes, scale, sel, dy, grad_gate, T: int, k: int, D: int):
+    check(lib, lib.amoe_gate_grad_codes(dtype_code(dy), _p(codes), _p(scale), _p(sel), int(sel.dtype == torch.int64),
+                                        _p(dy), _p(grad_gate), T, k, D, stream), "amoe_gate_grad_codes")
 
 
 def ksum(lib, stream, full, out, T: int, k: int, D: int):

@@ -239,10 +239,11 @@ def main():
 
     # HIP events around every launch, on the stream the kernels are launched on; a launch is named
     # by its op and its position among that op's calls within one step
-    ROLES = {"cvmm_fwd": ["fwd_up (gemm_rows_kernel, forward, K-tile split)", "fwd_down (gemm_rows_kernel, forward)"],
-             "cvmm_bwd_w": ["wgrad_down (gemm_wgrad_kernel)", "wgrad_up (gemm_wgrad_kernel)"],
-             "cvmm_bwd_x": ["xgrad_down (gemm_rows_kernel, input gradient)",
-                            "xgrad_up (gemm_rows_kernel, input gradient)"]}
+    ROLES = {"cvmm_fwd": ["fwd_up (up-projection forward)", "fwd_down (down-projection forward)"],
+             "cvmm_bwd_w": ["wgrad_down (weight gradient of the down-projection)",
+                            "wgrad_up (weight gradient of the up-projection)"],
+             "cvmm_bwd_x": ["xgrad_down (input gradient of the down-projection)",
+                            "xgrad_up (input gradient of the up-projection)"]}
     events = {}
     counter = {}
 
@@ -276,7 +277,7 @@ def main():
     # pass 1 (eager): HIP events around every launch give the per-launch durations
     saved = {}
     for name in ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x", "prepare_sel", "gate_reduce", "gate_grad", "ksum",
-                 "weight_abs_max", "segment_sum"):
+                 "weight_abs_max", "segment_sum", "gate_reduce_codes", "gate_grad_codes"):
         saved[name], w = timed(name)
         setattr(ops, name, w)
     torch.cuda.synchronize()

@@ -133,6 +133,13 @@ typedef struct amoe_fwd_args {
   float xq_inp_res;              /* its quantisation step, > 0 */
   int32_t x_is_quantized;        /* != 0: x is such an image made with this call's ir / inp_res:
                                     the input stage is skipped, the rescale is not */
+  /* The result as ADC codes (no counterpart in the reference): with an output quantiser, one K-tile and one
+     max |W| per expert, every result is (code * step[e]) * ir[e] with an integer code in [-half, half],
+     half = max(out_res, 1 / out_res) / 2 <= 127.  A caller that only streams the result once more (the gate
+     reduction, the gate gradient) can take it at a quarter of fp32 / half of bf16: */
+  uint8_t* code_out;             /* optional [n_out_rows, N]: code + 128; `out` is then not written and may be NULL */
+  int64_t ldcode;
+  float* code_scale_out;         /* with code_out: [E, 2] = (step[e], ir[e]); written for experts that have rows */
 } amoe_fwd_args;
 
 int amoe_cvmm_fwd(const amoe_fwd_args* args, void* stream);
@@ -234,6 +241,14 @@ int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, 
 /* grad_gate[t*k + j] = <z[t*k + j, :], dy[t, :]>   (cvmm.py:889) */
 int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate,
                    int64_t T, int32_t k, int32_t D, void* stream);
+/* amoe_gate_reduce / amoe_gate_grad on a result stored as ADC codes (amoe_fwd_args.code_out): row r = t*k + j
+ * belongs to expert sel[r] (the unsorted ids, int32 or int64), z[r, :] = ((code[r, :] - 128) * scale[e][0]) * scale[e][1]. */
+int amoe_gate_reduce_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel,
+                           int32_t sel_is_i64, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
+                           void* stream);
+int amoe_gate_grad_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel,
+                         int32_t sel_is_i64, const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D,
+                         void* stream);
 /* abs_max[r] = max_n |x[r, n]|                 (cvmm.py:733, 737) */
 int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, int32_t K,
                      float* abs_max, void* stream);

@@ -76,6 +76,11 @@ CASES = {
     # 256-column interior tiles: the 128 x 256 forward kernel (plain, clip + quantise, ADC without noise)
     "bf16_wide_plain": (dict(T=90, D=256, E=3, F=256, k=2), dict(), "bf16", 2e-2),
     "bf16_wide_ir_quant": (dict(T=90, D=256, E=3, F=256, k=2), dict(ir=True, inp_res=1 / 127, decay=0.01), "bf16", 2e-2),
+    # two K-tiles of 256 columns with per-expert ranges: the 128 x 256 input-gradient kernel with its masks
+    "bf16_wide_split": (dict(T=90, D=512, E=3, F=256, k=2),
+                        dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0, out_res=254.0,
+                             decay=0.01), "bf16", 2e-2),
+    "bf16_wide_ir_only": (dict(T=90, D=256, E=3, F=256, k=2), dict(ir=True, decay=0.01), "bf16", 2e-2),
     "bf16_wide_adc": (dict(T=90, D=256, E=3, F=256, k=2),
                       dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, bounds_up=[0, 96, 256]), "bf16", 2e-2),
     "f32_interior_ir_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(ir=True, decay=0.01), "f32", 1e-5),
@@ -138,6 +143,11 @@ def test_generated_noise_interior_bf16(emu_ops, split):
 
 def test_bf16_dac_codes_next_to_rounding_ties(emu_ops):
     util.check_bf16_dac_codes_near_ties(emu_ops)
+
+
+@pytest.mark.parametrize("noisy", [False, True])
+def test_result_as_adc_codes(emu_ops, noisy):
+    util.check_result_as_codes(emu_ops, noisy=noisy, T=71)
 
 
 def test_companions(emu_ops):
@@ -221,6 +231,6 @@ def test_chained_projections(emu_ops, dtype, D, F, T):
 
 
 @pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 128, 128, 60), (torch.bfloat16, 128, 128, 60),
-                                         (torch.bfloat16, 72, 40, 60)])
+                                         (torch.bfloat16, 72, 40, 60), (torch.bfloat16, 256, 256, 200)])
 def test_clipped_input_for_the_weight_gradient(emu_ops, dtype, D, F, T):
     util.check_clipped_input_output(emu_ops, dtype=dtype, T=T, D=D, F=F)

@@ -107,9 +107,12 @@ def test_full_size_analog_layer(ops, name, T, D, E, F, k, routing, mis):
     cfg = ffn.FFNConfig(inp_res=RES, bounds_up=bu if ntu > 1 else None, bounds_down=bd if ntd > 1 else None,
                         out_bound=OUT_BOUND, out_res=OUT_RES, noise_std=NOISE, noise_up=noise_up, noise_down=noise_dn,
                         decay=decay, input_min_percentage=min_pct, gradient_relative=True, gradient_scale=1.0)
-    y, p1, z, perm, in_index, offsets, ir_up, ir_dn = ffn.ffn_forward(x, keys, values, ir, gate, idx, cfg)
+    y, p1, z, perm, in_index, offsets, z_scale, ir_up, ir_dn = ffn.ffn_forward(x, keys, values, ir, gate, idx, cfg)
     torch.cuda.synchronize()
     print("forward done", flush=True)
+    z_kept = z
+    if z.dtype == torch.uint8:                       # the k-head result was kept as ADC codes
+        z = ops.dequant_codes(z, z_scale, idx)
     ss = flat[perm.long()]
     assert torch.equal(ir_up, ir[0, :, :ntu]) and torch.equal(ir_dn, ir[1, :, :ntd])
 
@@ -131,7 +134,7 @@ def test_full_size_analog_layer(ops, name, T, D, E, F, k, routing, mis):
 
     # ---- backward
     grad_x, grad_keys, grad_values, grad_ir, grad_gate = ffn.ffn_backward(
-        dy, x, keys, values, gate, p1, z, perm, in_index, offsets, ir_up, ir_dn, cfg, True)
+        dy, x, keys, values, gate, idx, p1, z_kept, z_scale, perm, in_index, offsets, ir_up, ir_dn, cfg, True)
     torch.cuda.synchronize()
     print("backward done", flush=True)
     tok = torch.div(perm, k, rounding_mode="floor").long()

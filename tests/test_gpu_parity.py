@@ -106,6 +106,16 @@ def test_config2_paper_scale_layer(ops, dtype):
     print(errs)
 
 
+def test_wide_tiles_layer(ops):
+    """Several row tiles per expert and several work items per workgroup of the 128 x 256 kernels (forward and
+    input gradient): two K-tiles of 256 columns, per-expert ranges, DAC / ADC, injected noise, range decay."""
+    print("wide tiles", flush=True)
+    errs = _run_case(ops, dict(T=4096, D=512, E=8, F=256, k=2),
+                     dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0, out_res=254.0,
+                          noise=0.04, decay=0.01, input_min_percentage=0.9), "bf16", seed=0, by_expert=True)
+    print(errs)
+
+
 def test_generated_noise_matches_counter_oracle(ops):
     pr = util.make_problem(9, T=500, D=256, E=8, F=128, k=2)
     ir = torch.full((2, 8, 1), 2.0)
@@ -137,6 +147,12 @@ def test_generated_noise_interior(ops, dtype, split):
 def test_bf16_dac_codes_next_to_rounding_ties(ops):
     print("bf16 DAC codes next to rounding ties", flush=True)
     util.check_bf16_dac_codes_near_ties(ops, device="cuda", T=960)
+
+
+@pytest.mark.parametrize("noisy", [False, True])
+def test_result_as_adc_codes(ops, noisy):
+    print("result as ADC codes", noisy, flush=True)
+    util.check_result_as_codes(ops, device="cuda", noisy=noisy, T=3000, D=1024, F=256, E=8, k=4)
 
 
 def test_companions(ops):
@@ -171,7 +187,8 @@ def test_chained_projections(ops, dtype, D, F, T):
 
 @pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 256, 128, 700), (torch.bfloat16, 256, 128, 700),
                                          (torch.bfloat16, 256, 192, 700), (torch.bfloat16, 72, 40, 700),
-                                         (torch.bfloat16, 256, 256, 1000), (torch.bfloat16, 256, 512, 1000)])
+                                         (torch.bfloat16, 256, 256, 1000), (torch.bfloat16, 256, 512, 1000),
+                                         (torch.bfloat16, 512, 256, 3000)])
 def test_clipped_input_for_the_weight_gradient(ops, dtype, D, F, T):
     util.check_clipped_input_output(ops, device="cuda", dtype=dtype, T=T, D=D, F=F)
 

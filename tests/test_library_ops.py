@@ -41,12 +41,20 @@ def test_fake_shapes_of_the_fused_operators_and_their_autograd():
     gate = torch.empty(T, k, requires_grad=True, **m)
     idx = torch.empty(T, k, dtype=torch.int64, **m)
     cfg = ffn.FFNConfig(inp_res=1 / 127, bounds_up=[0, 32, 64])
-    y, p1, z, perm, in_index, offsets = torch.ops.amoe.ffn_fwd(x, keys, values, ir, gate, idx, *ffn.cfg_astuple(cfg))
-    assert y.shape == (T, D) and p1.shape == (T * k, Fs) and z.shape == (T * k, D)
+    y, p1, z, perm, in_index, offsets, z_scale = torch.ops.amoe.ffn_fwd(x, keys, values, ir, gate, idx,
+                                                                        *ffn.cfg_astuple(cfg))
+    assert y.shape == (T, D) and p1.shape == (T * k, Fs) and z.shape == (T * k, D) and z_scale.numel() == 0
     assert perm.shape == in_index.shape == (T * k,) and offsets.shape == (E + 1,) and perm.dtype == torch.int32
     y.sum().backward()
     for t in (x, keys, values, ir, gate):
         assert t.grad.shape == t.shape
+    # bf16, 256 output columns, output quantiser, no injected noise: the k-head result is kept as ADC codes
+    b = dict(device="meta", dtype=torch.bfloat16)
+    xb, kb, vb = torch.empty(T, 256, **b), torch.empty(E, 256, 32, **b), torch.empty(E, 32, 256, **b)
+    cfg = ffn.FFNConfig(inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise_std=0.04)
+    out = torch.ops.amoe.ffn_fwd(xb, kb, vb, torch.empty(2, E, 1, device="meta"), torch.empty(T, k, **b), idx,
+                                 *ffn.cfg_astuple(cfg))
+    assert out[2].dtype == torch.uint8 and out[2].shape == (T * k, 256) and out[6].shape == (E, 2)
 
 
 def _analog_layer(fused: bool, noise: float = 0.04):

@@ -235,6 +235,43 @@ def check_bf16_dac_codes_near_ties(ops, device="cpu", T=96):
     np.testing.assert_array_equal(np32(img), codes2)
 
 
+def check_result_as_codes(ops, device="cpu", T=150, D=256, F=128, E=3, k=2, noisy=True):
+    """A forward whose result leaves as ADC codes (one byte per value + two factors per expert): the values behind
+    the codes round to exactly the bf16 result of the ordinary call, and the gate reduction / gate gradient that
+    read the codes agree with those that read the values."""
+    pr = make_problem(29, T, F, E, D, k, dtype=torch.bfloat16)          # (a down-projection: [M, F] -> [M, D])
+    M = T * k
+    g = torch.Generator().manual_seed(2)
+    p1 = torch.relu(torch.randn(M, F, generator=g)).bfloat16().to(device)
+    values = (torch.randn(E, F, D, generator=g) / F ** 0.5).bfloat16().to(device)
+    idx, gate = pr["idx"].to(device), pr["gate"].to(device)
+    dy = torch.randn(T, D, generator=g).bfloat16().to(device)
+    ss, perm, in_index, offsets = ops.prepare_sel(idx, E, k)
+    ir = torch.linspace(0.6, 1.4, E).reshape(E, 1).to(device)
+    wmax = ops.weight_abs_max(values, False)
+    kw = dict(ir=ir, ir_by_expert=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, wmax=wmax,
+              noise_std=0.04 if noisy else 0.0, noise_seed=77)
+    assert ops.codes_supported(p1, values, ir_by_expert=True, inp_res=1 / 127, n_tiles=1, out_bound=12.0,
+                               out_res=254.0, noise=None, per_channel=False)
+    z = ops.cvmm_fwd(p1, values, ss, offsets, perm, None, M, **kw)
+    codes, scale = ops.cvmm_fwd(p1, values, ss, offsets, perm, None, M, want_codes=True, **kw)
+    assert codes.dtype == torch.uint8 and tuple(codes.shape) == (M, D) and tuple(scale.shape) == (E, 2)
+    zf = ops.dequant_codes(codes, scale, idx)
+    assert torch.equal(zf.to(torch.bfloat16), z)
+    c = codes.cpu().numpy().astype(np.int32) - 128
+    assert np.abs(c).max() <= 127 and np.abs(c).max() > 20
+    # gate reduction and gate gradient from the codes: against float64 on the exact values, and close to the
+    # kernels that read the bf16 values
+    y = ops.gate_reduce_codes(codes, scale, idx, gate)
+    want_y = (gate.double().unsqueeze(-1) * zf.double().view(T, k, D)).sum(1)
+    assert rel_err(np32(y), want_y.cpu().numpy()) < 1e-2
+    assert rel_err(np32(y), np32(ops.gate_reduce(z, gate))) < 2e-2
+    gg = ops.gate_grad_codes(codes, scale, idx, dy, k)
+    want_gg = torch.einsum("tkd,td->tk", zf.double().view(T, k, D), dy.double())
+    assert rel_err(np32(gg), want_gg.cpu().numpy()) < 1e-2
+    assert rel_err(np32(gg), np32(ops.gate_grad(z, dy, k))) < 2e-2
+
+
 def check_row_chunked_wgrad(ops, device="cpu", dtype=torch.float32, T=600, D=136, F=72):
     """The weight gradient with the rows of an expert shared between workgroups (skewed routing: one
     heavy expert, one empty one) against the oracle, and its run-to-run determinism."""
