@@ -266,3 +266,127 @@ def test_full_size_bf16_dac_codes_exact(ops, name, T, D, E, F, k, routing, mis):
     mism = int((img.double() != want).sum())
     assert mism == 0, f"{mism} of {img.numel()} codes differ"
     assert float(want.abs().max()) == 127.0 and int((want == 0).sum()) < want.numel()
+
+
+# ------------------------------------------------------------------------------- the layer inside its caller
+def _decoder(cfgmod, *, vocab, d_model, n_layers, n_heads, context, E, F, k, noise=NOISE, dtype=torch.bfloat16):
+    from analog_moe_amd.decoder import SigmaMoEDecoder
+    from analog_moe_amd.moe_layer import AnalogSigmaMoELayer
+
+    def make(i):
+        r = cfgmod.TorchInferenceRPUConfig()
+        r.forward.inp_res = r.forward.out_res = 2 ** 8 - 2
+        r.forward.out_bound = OUT_BOUND
+        r.forward.out_noise = noise
+        ir = r.pre_post.input_range
+        ir.enable, ir.learn_input_range, ir.init_value, ir.decay = True, True, 3.0, 0.01
+        return AnalogSigmaMoELayer(r, d_model=d_model, n_experts=E, expert_size=F, k=k)
+    torch.manual_seed(0)
+    model = SigmaMoEDecoder(vocab, d_model, n_layers, n_heads, context, make).cuda().to(dtype)
+    model.train()
+    for blk in model.blocks:
+        blk.ffn.use_device_noise_counter()
+    return model
+
+
+def test_config5_full_size_training_step():
+    """BASELINE configuration 5 at full size: one training step (and a second one after the optimizer update) of the
+    16-layer decoder -- d_model 1024, 16 heads, 64 experts x 256, k = 8, context 1024, batch 16, vocabulary 8000,
+    bf16, 8-bit DAC / ADC, output noise drawn in the kernels, learned input ranges.  The loss is finite, every
+    parameter of every block gets a finite gradient, and the feed-forward of a middle block returns exactly what
+    the stand-alone layer computes from the captured input under the same noise seed."""
+    from analog_moe_amd import config as cfgmod
+    print("config 5, full size", flush=True)
+    V, D, L, H, S, B = 8000, 1024, 16, 16, 1024, 16
+    model = _decoder(cfgmod, vocab=V, d_model=D, n_layers=L, n_heads=H, context=S, E=64, F=256, k=8)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, V, (B, S), generator=g).cuda()
+    labels = torch.roll(ids, -1, dims=1)
+    ffn = model.blocks[7].ffn
+    seen = {}
+    h0 = ffn.register_forward_pre_hook(lambda m, a: seen.update(counter=m.noise_counter.clone()))
+    h1 = ffn.register_forward_hook(lambda m, a, out: seen.update(x=a[0].detach(), y=out[0].detach(),
+                                                                 reg=out[1].detach()))
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+    loss, reg = model(ids, labels, reg_weight=0.01)
+    h0.remove()
+    h1.remove()
+    assert torch.isfinite(loss) and torch.isfinite(reg)
+    assert abs(float(loss.detach()) - float(np.log(V))) < 1.0          # random initialisation: about log(vocabulary)
+    loss.backward()
+    missing = [n for n, p in model.named_parameters() if p.requires_grad and p.grad is None]
+    assert missing == []
+    bad = [n for n, p in model.named_parameters() if p.grad is not None and not bool(torch.isfinite(p.grad).all())]
+    assert bad == []
+    dead = [n for n, p in model.named_parameters()
+            if p.grad is not None and ("keys" in n or "values" in n) and float(p.grad.abs().max()) == 0.0]
+    assert dead == []
+    # the block's feed-forward against the stand-alone layer: same input, same noise seed word
+    assert seen["x"].shape == (B, S, D)
+    after = ffn.noise_counter.clone()
+    ffn.noise_counter.copy_(seen["counter"])
+    with torch.no_grad():
+        alone, reg_alone = ffn(seen["x"])
+    assert torch.equal(ffn.noise_counter, after)
+    assert torch.equal(alone, seen["y"]) and torch.equal(reg_alone, seen["reg"])
+    opt.step()
+    model.post_update_step()
+    opt.zero_grad(set_to_none=True)
+    loss2, _ = model(ids, labels, reg_weight=0.01)
+    assert torch.isfinite(loss2) and float(loss2.detach()) < float(loss.detach()) + 0.5
+    torch.cuda.synchronize()
+
+
+def test_decoder_step_in_a_hip_graph_matches_eager_steps():
+    """The whole training step (forward, loss, backward, AdamW, weight clipping) captured once and replayed: every
+    replay's loss against the loss of the same step launched eagerly from the same initial state.  The noise
+    seeds advance in device memory, so both sequences draw the same noise; what differs is the order of
+    atomic additions in stock PyTorch kernels (embedding gradients), hence the tolerance."""
+    from analog_moe_amd import config as cfgmod
+    print("decoder step in a HIP graph", flush=True)
+    kw = dict(vocab=211, d_model=256, n_layers=2, n_heads=4, context=64, E=8, F=256, k=2)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, 211, (16, 64), generator=g).cuda()
+    labels = torch.roll(ids, -1, dims=1)
+
+    def steps(graph, n=6, warm=3):
+        model = _decoder(cfgmod, **kw)
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-3, capturable=True)
+
+        def step():
+            loss, _ = model(ids, labels, reg_weight=0.01)
+            loss.backward()
+            opt.step()
+            model.post_update_step()
+            return loss.detach()
+        out = []
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warm):
+                opt.zero_grad(set_to_none=True)
+                out.append(float(step()))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        if not graph:
+            for _ in range(n):
+                opt.zero_grad(set_to_none=True)
+                out.append(float(step()))
+            return out
+        cg = torch.cuda.CUDAGraph()
+        opt.zero_grad(set_to_none=True)
+        with torch.cuda.graph(cg):
+            captured = step()
+        for i in range(n - 1):           # (the capture itself does not run the step)
+            cg.replay()
+            torch.cuda.synchronize()
+            out.append(float(captured))
+            _ = torch.randn(64, 64, device="cuda").sum().item()      # eager work between the replays
+        return out
+    eager = steps(False)
+    replayed = steps(True)
+    print(eager, replayed)
+    assert all(np.isfinite(eager)) and all(np.isfinite(replayed))
+    assert eager[-1] < eager[0]
+    for a, b in zip(eager[:len(replayed)], replayed):
+        assert abs(a - b) < 2e-2 * abs(a), (eager, replayed)
