@@ -51,9 +51,9 @@ inline int num_compute_units() {
 // would otherwise get more work items than its descriptor table holds, rounded up to a multiple
 // of the column-block count (so that the column blocks of one row tile run side by side), never
 // more than there are work items.
-inline int persistent_grid(int row_tiles, int col_blocks) {
+inline int persistent_grid(int row_tiles, int col_blocks, int per_cu = 2) {
   const long long work = (long long)row_tiles * col_blocks;
-  long long g = 2LL * num_compute_units();
+  long long g = (long long)per_cu * num_compute_units();
   const long long need = (work + kMaxDesc - 1) / kMaxDesc;
   if (need > g) g = need;
   if (g % col_blocks) g += col_blocks - g % col_blocks;
@@ -109,26 +109,32 @@ int launch_fwd256_as(const RowsParams& p, int grid, hipStream_t st) {
 
 // The 128 x 256 input-gradient kernel, for the same launches (and column tiles that are multiples of 256).  The
 // partial sums of the input-range gradient then cover 256 columns each; *n_count_blocks is the grid that ran.
-int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks) {
+template <int COLS>
+int launch_bwdx256_cols(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks) {
+  p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles, COLS);
+  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks, COLS == 128 ? 3 : 2);
+  *n_count_blocks = grid;
+  const bool relu = a->relu_mask != 0, xc = a->xc_out != nullptr;
+  if (a->x == nullptr) {
+    hipLaunchKernelGGL((&bwdx256_kernel<false, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+  } else if (!relu) {
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, false, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<true, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+  } else {
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, true, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<true, true, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+  }
+  return launch_rc();
+}
+
+int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks, int* block_cols) {
   if (!rows_all_interior(p, MODE_BWDX, kFBK)) return AMOE_EUNSUPPORTED;
   if (a->ir != nullptr && !a->ir_by_expert) return AMOE_EUNSUPPORTED;
   if (a->x != nullptr && (!aligned(a->x, 16) || a->ldx % 8)) return AMOE_EUNSUPPORTED;   // 16-byte pieces of x rows
   for (int t = 0; t < a->n_tiles; t++)
     if ((a->tile_bounds[t + 1] - a->tile_bounds[t]) % kFCols) return AMOE_EUNSUPPORTED;
-  p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles, kFCols);
-  const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
-  *n_count_blocks = grid;
-  const bool relu = a->relu_mask != 0, xc = a->xc_out != nullptr;
-  if (a->x == nullptr) {
-    hipLaunchKernelGGL((&bwdx256_kernel<false, false, false>), dim3(grid), dim3(kThreads), 0, st, p);
-  } else if (!relu) {
-    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, false, true>), dim3(grid), dim3(kThreads), 0, st, p);
-    else hipLaunchKernelGGL((&bwdx256_kernel<true, false, false>), dim3(grid), dim3(kThreads), 0, st, p);
-  } else {
-    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, true, true>), dim3(grid), dim3(kThreads), 0, st, p);
-    else hipLaunchKernelGGL((&bwdx256_kernel<true, true, false>), dim3(grid), dim3(kThreads), 0, st, p);
-  }
-  return launch_rc();
+  *block_cols = kFCols;
+  return launch_bwdx256_cols<kFCols>(p, a, st, n_count_blocks);
 }
 
 int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st) {
@@ -504,7 +510,9 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   p.xc_vec = a->xc_out && aligned(a->xc_out, 16) && (a->ldxc % CH == 0) && bounds_multiple_of(a->n_tiles, a->tile_bounds, CH);
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (use_ir) {
-    const size_t need = (size_t)p.n_col_blocks * a->M * sizeof(float) + (size_t)grid * sizeof(int32_t);
+    // (one count per workgroup; no grid is larger than the number of work items)
+    const size_t need = (size_t)p.n_col_blocks * a->M * sizeof(float) +
+                        (size_t)max_row_tiles(a->M, a->E) * p.n_col_blocks * sizeof(int32_t);
     if (a->workspace_bytes < need) return AMOE_EWORKSPACE;
     p.irg_partial = static_cast<float*>(a->workspace);
     p.notclip_count = reinterpret_cast<int32_t*>(p.irg_partial + (size_t)p.n_col_blocks * a->M);
@@ -520,8 +528,9 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   int block_cols = kTileCols, n_count_blocks = grid;
   int rc = AMOE_EUNSUPPORTED;
   if (a->dtype == AMOE_BF16) {
-    rc = launch_bwdx256(p, a, st, &n_count_blocks);
-    if (rc == AMOE_OK) block_cols = kFCols;
+    int cols = kTileCols;
+    rc = launch_bwdx256(p, a, st, &n_count_blocks, &cols);
+    if (rc == AMOE_OK) block_cols = cols;
   }
   if (rc == AMOE_EUNSUPPORTED)
     rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)

@@ -16,14 +16,18 @@ namespace amoe {
 // MASKS: the forward input is read for the clip mask against the input range (infinite if there is none) and, with
 // RELU, for the ReLU mask.  XC: also leave gate * clamp(x, +-ir) at the rows of x (needs MASKS).  The optional gate
 // scales the result in every variant.
-template <bool MASKS, bool RELU, bool XC>
-__global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p) {
+template <bool MASKS, bool RELU, bool XC, int COLS = kFCols>
+__global__ __launch_bounds__(kThreads, COLS == 128 ? 3 : 2) void bwdx256_kernel(const RowsParams p) {
   using T = uint16_t;
+  static_assert(COLS == 128 || COLS == 256, "output columns per workgroup tile");
   constexpr int BK = kFBK, CH = 8;
   constexpr int LDA = BK + 8, LDB = BK + 8;
-  constexpr int A_ELEMS = kTileRows * LDA, B_ELEMS = kFCols * LDB;
-  constexpr int STAGE = A_ELEMS + B_ELEMS;            // 15360 elements = 30 KB
-  constexpr int LDO = kFCols + 8;
+  constexpr int A_ELEMS = kTileRows * LDA, B_ELEMS = COLS * LDB;
+  constexpr int STAGE = A_ELEMS + B_ELEMS;            // 256 columns: 15360 elements = 30 KB
+  constexpr int NB = COLS / 64;                       // rows of W per thread and step; 32-column blocks per wave
+  constexpr int WCOLS = COLS / 2;                     // columns per wave
+  constexpr int CPR = COLS / CH, RPP = kThreads / CPR;   // 16-byte pieces per row of a staged half tile; rows per pass
+  constexpr int LDO = COLS + 8;
   constexpr int HALF_ROWS = 64;
   constexpr int HALF = HALF_ROWS * LDO;               // one staged half tile: 33 KB
   constexpr int LDS_ELEMS = (2 * STAGE > 2 * HALF) ? 2 * STAGE : 2 * HALF;
@@ -128,29 +132,29 @@ __global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p
       if (MASKS) sXrow[tid] = n_xrow;
     }
     fetch_rows(it + 1);
-    const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb, kFCols);
+    const ColBlock colb = find_col_block(p.col_bounds, p.n_col_tiles, cb, COLS);
     const int c0 = colb.c0;
     const T* __restrict__ W = static_cast<const T*>(p.w) + (int64_t)e * p.w_se;
     const BufRsrc rsrcW = make_rsrc(W);
-    uint32_t w_off[4];
+    uint32_t w_off[NB];
 #pragma unroll
-    for (int i = 0; i < 4; i++) w_off[i] = (uint32_t)(((int64_t)(c0 + a_row + 64 * i) * p.w_snd + a_chunk * CH) * 2);
+    for (int i = 0; i < NB; i++) w_off[i] = (uint32_t)(((int64_t)(c0 + a_row + 64 * i) * p.w_snd + a_chunk * CH) * 2);
 
-    f32x16 acc[4][2];
+    f32x16 acc[NB][2];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < NB; a++)
 #pragma unroll
       for (int b = 0; b < 2; b++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
 
     const int nsteps = p.KD / BK;
-    Raw ra[2], rb[4];
+    Raw ra[2], rb[NB];
     auto load_step = [&](int s) {
 #pragma unroll
       for (int i = 0; i < 2; i++) ra[i] = buffer_load_b128(rsrcA, a_off[i], s * (BK * 2));
 #pragma unroll
-      for (int i = 0; i < 4; i++) rb[i] = buffer_load_b128(rsrcW, w_off[i], s * (BK * 2));
+      for (int i = 0; i < NB; i++) rb[i] = buffer_load_b128(rsrcW, w_off[i], s * (BK * 2));
     };
     auto store_step = [&](int buf) {
       T* __restrict__ dA = sStage + buf * STAGE;
@@ -158,30 +162,31 @@ __global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p
 #pragma unroll
       for (int i = 0; i < 2; i++) *reinterpret_cast<Raw*>(&dA[(a_row + 64 * i) * LDA + a_chunk * CH]) = ra[i];
 #pragma unroll
-      for (int i = 0; i < 4; i++) *reinterpret_cast<Raw*>(&dB[(a_row + 64 * i) * LDB + a_chunk * CH]) = rb[i];
+      for (int i = 0; i < NB; i++) *reinterpret_cast<Raw*>(&dB[(a_row + 64 * i) * LDB + a_chunk * CH]) = rb[i];
     };
     auto multiply_group = [&](const T* __restrict__ cA, const T* __restrict__ cB, int kk) {
-      u32x4 xf[2], wf[4];
+      u32x4 xf[2], wf[NB];
 #pragma unroll
       for (int ti = 0; ti < 2; ti++)
         xf[ti] = *reinterpret_cast<const u32x4*>(&cA[(wr * 64 + ti * 32 + l32) * LDA + kk + 8 * lh]);
 #pragma unroll
-      for (int fi = 0; fi < 4; fi++)
-        wf[fi] = *reinterpret_cast<const u32x4*>(&cB[(wc * 128 + fi * 32 + l32) * LDB + kk + 8 * lh]);
+      for (int fi = 0; fi < NB; fi++)
+        wf[fi] = *reinterpret_cast<const u32x4*>(&cB[(wc * WCOLS + fi * 32 + l32) * LDB + kk + 8 * lh]);
 #pragma unroll
-      for (int fi = 0; fi < 4; fi++)
+      for (int fi = 0; fi < NB; fi++)
 #pragma unroll
         for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
     };
-    // the forward-input rows of one half of the tile: 64 rows x 32 chunks, 8 per thread (rows tid / 32 + 8 i)
-    Raw xr[MASKS ? 8 : 1];
+    // the forward-input rows of one half of the tile: 64 rows x CPR pieces, 64 / RPP per thread (rows tid / CPR + RPP i)
+    constexpr int NX = HALF_ROWS / RPP;
+    Raw xr[MASKS ? NX : 1];
     auto load_x_half = [&](int h) {
       if constexpr (MASKS) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const int rl = (tid >> 5) + 8 * i;
+        for (int i = 0; i < NX; i++) {
+          const int rl = tid / CPR + RPP * i;
           const int rt = (rl >> 5) * 64 + h * 32 + (rl & 31);
-          const Raw* src = reinterpret_cast<const Raw*>(XF + (int64_t)sXrow[rt] * p.ldxf + c0 + (tid & 31) * CH);
+          const Raw* src = reinterpret_cast<const Raw*>(XF + (int64_t)sXrow[rt] * p.ldxf + c0 + (tid % CPR) * CH);
           // (with the clipped input written back, every row of x belongs to one sorted position: read once)
           xr[i] = XC ? __builtin_nontemporal_load(src) : *src;
         }
@@ -190,8 +195,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p
     auto park_x_half = [&](T* __restrict__ sX) {
       if constexpr (MASKS) {
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-          *reinterpret_cast<Raw*>(&sX[((tid >> 5) + 8 * i) * LDO + (tid & 31) * CH]) = xr[i];
+        for (int i = 0; i < NX; i++)
+          *reinterpret_cast<Raw*>(&sX[(tid / CPR + RPP * i) * LDO + (tid % CPR) * CH]) = xr[i];
       }
     };
 
@@ -235,10 +240,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p
         const uint64_t valid_lanes = wave_ballot(valid);
         float part = 0.f;
 #pragma unroll
-        for (int fi = 0; fi < 4; fi++) {
+        for (int fi = 0; fi < NB; fi++) {
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const int cl = wc * 128 + fi * 32 + 8 * q + 4 * lh;
+            const int cl = wc * WCOLS + fi * 32 + 8 * q + 4 * lh;
             float v[4];
             if constexpr (MASKS) {
               float xv[4];
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwdx256_kernel(const RowsParams p
       if (MASKS && h == 0) load_x_half(1);        // in flight while the first half leaves
       __syncthreads();
       {
-        constexpr int OCPR = kFCols / CH, ORPP = kThreads / OCPR;      // 32 chunks per row, 8 rows per pass
+        constexpr int OCPR = CPR, ORPP = RPP;
 #pragma unroll
         for (int i0 = 0; i0 < HALF_ROWS / ORPP; i0 += 4) {
           Raw seg[4], segx[XC ? 4 : 1];

@@ -42,12 +42,15 @@ template <typename T>
 __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradParams p) {
   using EL = Elem<T>;
   constexpr int CH = EL::kChunk, MMAK = EL::kMmaK;
-  constexpr int BT = EL::kBK;                     // tokens per step
+  // tokens per step: 32 for both types.  (bf16 with 64 fills the LDS budget of two workgroups per CU; with 32 four
+  // fit, and the kernel, which waits on gathered rows more than on the matrix unit, runs about a tenth faster)
+  constexpr int BT = 32;
   constexpr int LD = kTileCols + EL::kPadRC;
   constexpr int STAGE = BT * LD;
   constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;
   constexpr bool IS_BF16 = sizeof(T) == 2;
-  static_assert(BT == 4 * RPP, "staging expects 4 passes");
+  constexpr int NP = BT / RPP;                    // staging passes per step
+  static_assert(BT == NP * RPP && 4 * BT <= kThreads, "whole staging passes; one metadata lane per row and item");
 
   constexpr int LDO = kTileCols + 16 / (int)sizeof(T);       // staged output tile, rows of 128 + 16 bytes
   static_assert(kTileRows * LDO <= 4 * STAGE, "the output tile must fit the stage buffers");
@@ -62,8 +65,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   // Workgroup ids go to the 8 XCDs round-robin.  All tiles of one chunk of rows run on one XCD
   // (they share those rows through that L2) and consecutive chunks / experts go to different
   // XCDs, so that a few heavy experts -- skewed routing -- do not pile up behind one L2.
-  // (scratch for the chunk search and the arrival flag lives in the stage buffers, which are idle
-  // then: the two stages fill the LDS budget of two workgroups per CU to the byte)
+  // (scratch for the chunk search and the arrival flag lives in the stage buffers, which are idle then)
   int* const sScanA = reinterpret_cast<int*>(sS);
   int* const sScanB = sScanA + 4;
   int* const sFound = sScanA + 8;
@@ -166,10 +168,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
     if (m_item < 4) meta(buf, m_row)[m_item] = m_val;
   };
 
-  Raw rx[4], rg[4];
+  Raw rx[NP], rg[NP];
   auto load_step = [&](int i0, int mbuf) {   // global -> registers, any shape; rows from the metadata
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NP; i++) {
       const int j = tid / CPR + RPP * i;
       const bool ok = i0 + j < seg1;
       const int* m = meta(mbuf, j);
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
   const uint32_t g_col_bytes = (uint32_t)((n0 + chunk * CH) * (int)sizeof(T));
   auto load_fast = [&](int mbuf) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NP; i++) {
       const int* m = meta(mbuf, tid / CPR + RPP * i);
       rx[i] = buffer_load_b128(rsX, (uint32_t)m[0] * x_row_bytes + x_col_bytes, 0);
       rg[i] = buffer_load_b128(rsG, (uint32_t)m[1] * g_row_bytes + g_col_bytes, 0);
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
     T* __restrict__ dG = sG + buf * STAGE;
     if (has_ir || GS != nullptr) {           // one branch for the whole step; a stage that is off is neutral
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
+      for (int i = 0; i < NP; i++) {
         const int* m = meta(mbuf, tid / CPR + RPP * i);
         const float scale = as_f32((uint32_t)m[2]), rng = as_f32((uint32_t)m[3]);
         float v[CH];
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NP; i++) {
       const int j = tid / CPR + RPP * i;
       *reinterpret_cast<Raw*>(&dX[j * LD + chunk * CH]) = rx[i];
       *reinterpret_cast<Raw*>(&dG[j * LD + chunk * CH]) = rg[i];

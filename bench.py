@@ -38,10 +38,9 @@ CONFIGS = {
                     "k=8, context 1024, batch 16, vocab 8000, bf16"),
 }
 PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a 256 MiB copy), from
-# the counter runs summarised under profiles/; None where not measured
-TRAFFIC = {"c3": {"fwd_up": 518229781, "fwd_down": 440371620, "wgrad_down": 370374685, "wgrad_up": 370383451,
-                  "xgrad_down": 478628453, "xgrad_up": 640301186}}
+# roofline.traffic (HBM bytes of the dominant launch) comes from profiles/bench_<config>_hbm_traffic.json, written by
+# bench_traffic.py from two rocprofv3 counter runs of this file; it is null when no such run is recorded or the
+# kernel sources changed after it.
 
 
 def cpu_baseline(cfg, pr, budget_tokens):
@@ -352,7 +351,9 @@ def main():
     gemm_flops = 2.0 * M * D * F                  # algorithmic flops of one launch of any of them
     achieved = gemm_flops / (kern[dom] * 1e-3)
     peak = PEAK[cfg["dtype"]]
-    traffic = TRAFFIC.get(args.config, {}).get(dom.split(" ")[0])
+    from bench_traffic import load_traffic
+    recorded, traffic_note = load_traffic(args.config)
+    traffic = None if recorded is None else recorded.get(dom.split(" ")[0])
     out = {
         "metric": "analog MoE layer fwd+bwd tokens/sec on 1 GPU; % of MFMA peak TFLOP/s",
         "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -369,7 +370,8 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom,
                      "achieved": achieved / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": traffic,
-                     "flops_per_launch": gemm_flops, "avg_launch_ms": kern[dom]},
+                     "flops_per_launch": gemm_flops, "avg_launch_ms": kern[dom],
+                     **({} if traffic_note is None else {"traffic_note": traffic_note})},
         "launch_ms": {n: round(v, 4) for n, v in sorted(kern.items(), key=lambda kv: -kv[1])},
         "gemm_frac_of_peak": {n.split(" ")[0]: round(gemm_flops / (kern[n] * 1e-3) / peak, 4) for n in gemms},
     }

@@ -1,0 +1,132 @@
+"""HBM bytes per launch of the six GEMM launches of a bench.py step, from two rocprofv3 counter runs.
+
+  cd /tmp; export TMPDIR=/tmp; cd <repository>
+  rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/prof/fetch -- python3 bench.py --steps 3 --warmup 1 \
+      --no-cpu-baseline --no-graph --copy-calibration
+  rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/prof/write -- python3 bench.py --steps 3 --warmup 1 \
+      --no-cpu-baseline --no-graph --copy-calibration
+  python3 bench_traffic.py gpurun_out/prof/fetch gpurun_out/prof/write --config c3
+
+writes profiles/bench_<config>_hbm_traffic.json (read by bench.py for roofline.traffic) and prints the table kept
+next to it as text.  Both counters are in KiB per dispatch; each is scaled by what it reads for the one 256 MiB
+device-to-device copy that --copy-calibration issues first.  The JSON carries a digest of the kernel sources: bench.py
+reports no traffic figure when the sources have changed since the counters were read.
+"""
+import argparse
+import csv
+import glob
+import hashlib
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(ROOT, "analog_moe_amd", "csrc")
+COPY_BYTES = 256 << 20
+ROLES = {"fwd": ("fwd_up", "fwd_down"), "xgrad": ("xgrad_down", "xgrad_up"), "wgrad": ("wgrad_down", "wgrad_up")}
+
+
+def source_digest() -> str:
+    """sha256 over the kernel sources (names and contents), the same for the profiling run and for bench.py"""
+    h = hashlib.sha256()
+    for dirpath, _, files in sorted(os.walk(CSRC)):
+        for f in sorted(files):
+            if f.endswith((".h", ".hip")):
+                h.update(f.encode())
+                with open(os.path.join(dirpath, f), "rb") as fh:
+                    h.update(fh.read())
+    return h.hexdigest()
+
+
+def traffic_file(config: str) -> str:
+    return os.path.join(ROOT, "profiles", f"bench_{config}_hbm_traffic.json")
+
+
+def load_traffic(config: str):
+    """(bytes per launch by role, note): the figures, or None and the reason there are none."""
+    path = traffic_file(config)
+    if not os.path.exists(path):
+        return None, "no counter run recorded for this workload"
+    with open(path) as fh:
+        rec = json.load(fh)
+    if rec.get("source_digest") != source_digest():
+        return None, "the kernel sources changed after the recorded counter run"
+    return {role: v["total_bytes"] for role, v in rec["launches"].items()}, None
+
+
+def family(kernel: str):
+    """Which of the three GEMM families a kernel name belongs to (None: a companion)."""
+    if "fwd256_kernel" in kernel:
+        return "fwd"
+    if "bwdx256_kernel" in kernel:
+        return "xgrad"
+    if "gemm_wgrad_kernel" in kernel:
+        return "wgrad"
+    if "gemm_rows_kernel<" in kernel:            # <T, W_KC, MODE, FAST>: mode 2 is the input gradient
+        args = kernel.split("gemm_rows_kernel<", 1)[1].split(">", 1)[0].split(",")
+        return "xgrad" if args[2].strip() == "2" else "fwd"
+    return None
+
+
+def read_counter(directory: str, counter: str):
+    """Per role: list of counter readings (one per step); and the copy's reading."""
+    files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+        sys.exit(f"no *counter_collection.csv under {directory}")
+    with open(files[0]) as fh:
+        rows = [r for r in csv.DictReader(fh) if r["Counter_Name"] == counter]
+    rows.sort(key=lambda r: int(r.get("Dispatch_Id", 0)))
+    seen = {"fwd": 0, "xgrad": 0, "wgrad": 0}
+    out, copy, kernels = {}, None, {}
+    for r in rows:
+        name, val = r["Kernel_Name"], float(r["Counter_Value"])
+        if "copyBuffer" in name:
+            copy = val if copy is None else max(copy, val)
+            continue
+        fam = family(name)
+        if fam is None:
+            continue
+        role = ROLES[fam][seen[fam] % 2]
+        seen[fam] += 1
+        out.setdefault(role, []).append(val)
+        kernels[role] = name.split("(")[0].replace("void ", "")
+    if copy is None:
+        sys.exit(f"no device copy in {directory}: run bench.py with --copy-calibration")
+    return out, copy, kernels
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("fetch_dir")
+    ap.add_argument("write_dir")
+    ap.add_argument("--config", default="c3")
+    ap.add_argument("--skip-first", type=int, default=1, help="steps at the start (warm-up) left out of the average")
+    args = ap.parse_args()
+    fetch, fcopy, kernels = read_counter(args.fetch_dir, "FETCH_SIZE")
+    write, wcopy, _ = read_counter(args.write_dir, "WRITE_SIZE")
+    fscale, wscale = COPY_BYTES / (fcopy * 1024.0), COPY_BYTES / (wcopy * 1024.0)
+    launches = {}
+    print(f"copy of {COPY_BYTES >> 20} MiB reads FETCH_SIZE {fcopy:.0f}, WRITE_SIZE {wcopy:.0f} (KiB): "
+          f"scale factors fetch x{fscale:.3f}, write x{wscale:.3f}")
+    print(f"{'launch':12s} {'FETCH_SIZE':>11s} {'WRITE_SIZE':>11s} {'read MB':>9s} {'write MB':>9s} {'total MB':>9s}  kernel")
+    for fam in ("fwd", "xgrad", "wgrad"):
+        for role in ROLES[fam]:
+            f = fetch[role][args.skip_first:] or fetch[role]
+            w = write[role][args.skip_first:] or write[role]
+            fk, wk = sum(f) / len(f), sum(w) / len(w)
+            rb, wb = fk * 1024.0 * fscale, wk * 1024.0 * wscale
+            launches[role] = {"fetch_size_kib": fk, "write_size_kib": wk, "read_bytes": rb, "write_bytes": wb,
+                              "total_bytes": rb + wb, "kernel": kernels[role]}
+            print(f"{role:12s} {fk:11.0f} {wk:11.0f} {rb / 1e6:9.1f} {wb / 1e6:9.1f} {(rb + wb) / 1e6:9.1f}  {kernels[role]}")
+    rec = {"workload": args.config, "source_digest": source_digest(),
+           "copy_calibration": {"bytes": COPY_BYTES, "fetch_size_kib": fcopy, "write_size_kib": wcopy,
+                                "fetch_scale": fscale, "write_scale": wscale},
+           "launches": launches}
+    with open(traffic_file(args.config), "w") as fh:
+        json.dump(rec, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print("wrote", os.path.relpath(traffic_file(args.config), ROOT))
+
+
+if __name__ == "__main__":
+    main()
