@@ -42,9 +42,10 @@ template <typename T>
 __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradParams p) {
   using EL = Elem<T>;
   constexpr int CH = EL::kChunk, MMAK = EL::kMmaK;
-  // tokens per step: 32 for both types.  (bf16 with 64 fills the LDS budget of two workgroups per CU; with 32 four
-  // fit, and the kernel, which waits on gathered rows more than on the matrix unit, runs about a tenth faster)
-  constexpr int BT = 32;
+  // tokens per step.  (bf16: 64 fills the LDS budget of two workgroups per CU.  With 32, four fit and the kernel
+  // alone runs about a tenth faster, but it then leaves no registers for the row-wise kernels the layer runs next to
+  // it on a second stream, and the training step as a whole gets slower.)
+  constexpr int BT = EL::kBK;
   constexpr int LD = kTileCols + EL::kPadRC;
   constexpr int STAGE = BT * LD;
   constexpr int CPR = kTileCols / CH, RPP = kThreads / CPR;

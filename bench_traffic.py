@@ -73,7 +73,10 @@ def read_counter(directory: str, counter: str):
     files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
     if not files:
         sys.exit(f"no *counter_collection.csv under {directory}")
-    with open(files[0]) as fh:
+    files.sort(key=os.path.getmtime)
+    if len(files) > 1:
+        print(f"{len(files)} counter files under {directory}: reading the newest, {files[-1]}", file=sys.stderr)
+    with open(files[-1]) as fh:
         rows = [r for r in csv.DictReader(fh) if r["Counter_Name"] == counter]
     rows.sort(key=lambda r: int(r.get("Dispatch_Id", 0)))
     seen = {"fwd": 0, "xgrad": 0, "wgrad": 0}
