@@ -745,12 +745,13 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
   return launch_rc();
 }
 
-int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, float* out, void* stream) {
-  if (E < 1 || n_tiles < 1 || n_tiles > AMOE_MAX_TILES) return AMOE_EINVAL;
+int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, float* out, int64_t ldout,
+                     void* stream) {
+  if (E < 1 || n_tiles < 1 || n_tiles > AMOE_MAX_TILES || ldout < n_tiles) return AMOE_EINVAL;
   if (!v || !offsets || !out) return AMOE_ENULL;
   if (!aligned(v, 4) || !aligned(offsets, 4) || !aligned(out, 4)) return AMOE_EALIGN;
   hipLaunchKernelGGL(segment_sum_kernel, dim3(E, n_tiles), dim3(kThreads), 0, static_cast<hipStream_t>(stream), v,
-                     offsets, (int)n_tiles, out);
+                     offsets, (int)n_tiles, out, (long long)ldout);
   return launch_rc();
 }
 

@@ -310,7 +310,7 @@ __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __res
 // out[e, t] = sum_{i in [offsets[e], offsets[e+1])} v[i, t], one workgroup per (expert, tile).
 __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float* __restrict__ v,
                                                                 const int32_t* __restrict__ offsets, int n_tiles,
-                                                                float* __restrict__ out) {
+                                                                float* __restrict__ out, long long ldout) {
   __shared__ float red[4];
   const int e = blockIdx.x, t = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float* __re
   for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
   if (lane == 0) red[tid >> 6] = s;
   __syncthreads();
-  if (tid == 0) out[(long long)e * n_tiles + t] = (red[0] + red[1]) + (red[2] + red[3]);
+  if (tid == 0) out[(long long)e * ldout + t] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
 __device__ __forceinline__ double block_sum_double(double v, double* red /* LDS [4] */) {

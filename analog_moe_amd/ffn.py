@@ -137,7 +137,7 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
     by = dict(ir_by_expert=ir_up is not None)
     irkw = dict(gradient_relative=cfg.gradient_relative, gradient_scale=cfg.gradient_scale, decay=cfg.decay,
                 input_min_percentage=cfg.input_min_percentage)
-    tok = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
+    tok = in_index                               # token of each sorted position: perm // k, as the sort left it
     # the input gradient reads p1 for its masks anyway; it also leaves gate * clamp(p1), which is the
     # x operand of the weight gradient (otherwise every block of its output columns clips and scales)
     gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
@@ -164,9 +164,11 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
     grad_ir = None
     if ir_up is not None and want_ir_grad:
         ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
-        grad_ir = torch.zeros((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
-        grad_ir[0, :, :ntu] = ops.segment_sum(irg_up, offsets, E)
-        grad_ir[1, :, :ntd] = ops.segment_sum(irg_dn, offsets, E)
+        # the two tables of per-expert sums are written where they belong; only columns neither has need a zero
+        make = torch.empty if ntu == ntd else torch.zeros
+        grad_ir = make((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
+        ops.segment_sum(irg_up, offsets, E, out=grad_ir[0, :, :ntu])
+        ops.segment_sum(irg_dn, offsets, E, out=grad_ir[1, :, :ntd])
     return grad_x, grad_keys, grad_values, grad_ir, grad_gate
 
 

@@ -270,17 +270,20 @@ def weight_abs_max(w: torch.Tensor, per_channel: bool) -> torch.Tensor:
     return out
 
 
-def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int) -> torch.Tensor:
-    """out[e, t] = sum of v[i, t] over expert e's sorted rows."""
+def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[e, t] = sum of v[i, t] over expert e's sorted rows.  ``out``: fp32 [E, columns of v] to write into (its
+    rows may lie further apart than its columns: a slice of a wider table)."""
     _need_gpu(v, offsets)
     cols = 1
     for d in v.shape[1:]:
         cols *= d
     v2 = _f32c(v.reshape(v.shape[0], cols))       # (an explicit column count: v may have no rows)
+    if out is None:
+        out = torch.empty((n_experts, cols), dtype=torch.float32, device=v2.device)
     if v2.shape[0] == 0:                           # no sorted positions at all: nothing to read
-        return torch.zeros((n_experts, cols), dtype=torch.float32, device=v2.device)
-    out = torch.empty((n_experts, v2.shape[1]), dtype=torch.float32, device=v2.device)
-    raw.segment_sum(get_lib(), _stream(v2), v2, offsets, n_experts, v2.shape[1], out)
+        return out.zero_()
+    raw.segment_sum(get_lib(), _stream(v2), v2, offsets, n_experts, cols, out)
     return out
 
 

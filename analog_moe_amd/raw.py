@@ -237,8 +237,12 @@ def weight_abs_max(lib, stream, w, cols: int, out):
 
 
 def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out):
+    """out: fp32 [E, n_tiles], rows any stride apart (a slice of a wider table will do)"""
+    if (out.dtype != torch.float32 or out.dim() != 2 or tuple(out.shape) != (E, n_tiles) or
+            (n_tiles > 1 and out.stride(1) != 1) or out.stride(0) < n_tiles):
+        raise ValueError("out must be float32 [E, n_tiles] with unit column stride")
     check(lib, lib.amoe_segment_sum(_p(_f32(v, "v")), _p(_i32(offsets, "offsets")), E, n_tiles,
-                                    _p(_f32(out, "out")), stream), "amoe_segment_sum")
+                                    _p(out), out.stride(0), stream), "amoe_segment_sum")
 
 
 def expert_std(lib, stream, x, in_index, offsets, E: int, out):

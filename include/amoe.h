@@ -256,10 +256,11 @@ int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, in
  * (moe_layer_aihwkit_lightning.py:480-487) */
 int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N,
                         int32_t cols, float* wmax, void* stream);
-/* out[e, t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]
- * (moe_layer_aihwkit_lightning.py:447-448), fixed order. */
+/* out[e * ldout + t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]
+ * (moe_layer_aihwkit_lightning.py:447-448), fixed order.  ldout >= n_tiles: the row stride of out, so that the
+ * sums can land in a slice of a wider table. */
 int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles,
-                     float* out, void* stream);
+                     float* out, int64_t ldout, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Per-expert unbiased standard deviation of the routed rows' elements, for input-range
