@@ -8,7 +8,7 @@ from __future__ import annotations
 import ctypes as C
 
 AMOE_MAX_TILES = 16
-AMOE_F32, AMOE_BF16 = 0, 1
+AMOE_F32, AMOE_BF16, AMOE_F16 = 0, 1, 2
 P = C.c_void_p
 
 

@@ -296,7 +296,7 @@ int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, in
 // ------------------------------------------------------------------------------ forward
 int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
-  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16 && a->dtype != AMOE_F16) return AMOE_EINVAL;
   if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->n_in_rows < 0 || a->n_out_rows < 0) return AMOE_EINVAL;
   if (a->M == 0) return AMOE_OK;
   if (!a->x || !a->w || (!a->out && !a->code_out) || !a->offsets || !a->in_index) return AMOE_ENULL;
@@ -364,6 +364,8 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (a->dtype == AMOE_F32)
     return w_kc ? launch_rows<float, true>(p, mode, grid, st) : launch_rows<float, false>(p, mode, grid, st);
+  if (a->dtype == AMOE_F16)
+    return w_kc ? launch_rows<f16_t, true>(p, mode, grid, st) : launch_rows<f16_t, false>(p, mode, grid, st);
   return w_kc ? launch_rows<uint16_t, true>(p, mode, grid, st) : launch_rows<uint16_t, false>(p, mode, grid, st);
 }
 
@@ -404,7 +406,7 @@ size_t amoe_bwd_w_workspace(const amoe_bwd_w_args* a) {
 
 int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
-  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16 && a->dtype != AMOE_F16) return AMOE_EINVAL;
   if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->n_x_rows < 0 || a->n_g_rows < 0) return AMOE_EINVAL;
   if (!a->grad_w || !a->offsets) return AMOE_ENULL;
   if (a->M > 0 && (!a->x || !a->g || !a->in_index)) return AMOE_ENULL;
@@ -454,12 +456,20 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
       auto r = &wgrad_reduce_kernel<float>;
       hipLaunchKernelGGL(r, dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
     }
-  } else {
+  } else if (a->dtype == AMOE_BF16) {
     auto k = &gemm_wgrad_kernel<uint16_t>;
     hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
     if (int rc = launch_rc()) return rc;
     if (p.rows_per_chunk > 0) {
       auto r = &wgrad_reduce_kernel<uint16_t>;
+      hipLaunchKernelGGL(r, dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
+    }
+  } else {
+    auto k = &gemm_wgrad_kernel<f16_t>;
+    hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);
+    if (int rc = launch_rc()) return rc;
+    if (p.rows_per_chunk > 0) {
+      auto r = &wgrad_reduce_kernel<f16_t>;
       hipLaunchKernelGGL(r, dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
     }
   }
@@ -477,7 +487,7 @@ size_t amoe_bwd_x_workspace(int64_t M, int32_t K, int32_t n_tiles) {
 
 int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
-  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16 && a->dtype != AMOE_F16) return AMOE_EINVAL;
   if (a->M < 0 || a->N < 1 || a->K < 1 || a->E < 1 || a->E > kSelMaxExperts || a->n_g_rows < 0) return AMOE_EINVAL;
   if (a->M == 0) return AMOE_OK;
   if (!a->g || !a->w || !a->grad_x_full || !a->offsets || !a->g_index || !a->out_index) return AMOE_ENULL;
@@ -533,8 +543,9 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
     if (rc == AMOE_OK) block_cols = cols;
   }
   if (rc == AMOE_EUNSUPPORTED)
-    rc = a->dtype == AMOE_F32 ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
-                              : launch_rows<uint16_t, true>(p, MODE_BWDX, grid, st);
+    rc = a->dtype == AMOE_F32   ? launch_rows<float, true>(p, MODE_BWDX, grid, st)
+         : a->dtype == AMOE_F16 ? launch_rows<f16_t, true>(p, MODE_BWDX, grid, st)
+                                : launch_rows<uint16_t, true>(p, MODE_BWDX, grid, st);
   if (rc) return rc;
   if (use_ir) {
     IrFinalizeParams f{};
@@ -553,7 +564,7 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
 // ------------------------------------------------------------------------------ row-wise companions
 static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
                        void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
   if (T == 0) return AMOE_OK;
   if (!z || !y) return AMOE_ENULL;
@@ -569,10 +580,15 @@ static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, 
     auto kf = &head_reduce_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
                        static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D, vec);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &head_reduce_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
                        static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D,
+                       vec);
+  } else {
+    auto kf = &head_reduce_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(z),
+                       static_cast<const f16_t*>(gate), static_cast<f16_t*>(y), (long long)T, (int)k, (int)D,
                        vec);
   }
   return launch_rc();
@@ -590,7 +606,7 @@ int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, 
 
 int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D,
                    void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
   if (T == 0) return AMOE_OK;
   if (!z || !dy || !grad_gate) return AMOE_ENULL;
@@ -604,17 +620,21 @@ int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate
     auto kf = &gate_grad_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
                        static_cast<const float*>(dy), static_cast<float*>(grad_gate), (long long)T, (int)k, (int)D, vec);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &gate_grad_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
                        static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), (long long)T, (int)k, (int)D, vec);
+  } else {
+    auto kf = &gate_grad_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(z),
+                       static_cast<const f16_t*>(dy), static_cast<f16_t*>(grad_gate), (long long)T, (int)k, (int)D, vec);
   }
   return launch_rc();
 }
 
 static int codes_args_ok(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel, int32_t sel_is_i64,
                          const void* a, const void* b, int64_t T, int32_t k, int32_t D) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
   if (D % 16) return AMOE_EUNSUPPORTED;
   if (T == 0) return AMOE_OK;
@@ -636,10 +656,14 @@ int amoe_gate_reduce_codes(int32_t dtype, const uint8_t* codes, const float* sca
     auto kf = &head_reduce_codes_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
                        static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &head_reduce_codes_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
                        static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D);
+  } else {
+    auto kf = &head_reduce_codes_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const f16_t*>(gate), static_cast<f16_t*>(y), (long long)T, (int)k, (int)D);
   }
   return launch_rc();
 }
@@ -655,17 +679,21 @@ int amoe_gate_grad_codes(int32_t dtype, const uint8_t* codes, const float* scale
     auto kf = &gate_grad_codes_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
                        static_cast<const float*>(dy), static_cast<float*>(grad_gate), (long long)T, (int)k, (int)D);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &gate_grad_codes_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
                        static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(grad_gate), (long long)T, (int)k, (int)D);
+  } else {
+    auto kf = &gate_grad_codes_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
+                       static_cast<const f16_t*>(dy), static_cast<f16_t*>(grad_gate), (long long)T, (int)k, (int)D);
   }
   return launch_rc();
 }
 
 int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, int32_t K, float* abs_max,
                      void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (rows < 0 || K < 1 || ldx < K) return AMOE_EINVAL;
   if (rows == 0) return AMOE_OK;
   if (!x || !abs_max) return AMOE_ENULL;
@@ -677,9 +705,13 @@ int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, in
     auto kf = &row_abs_max_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(x),
                        (long long)ldx, (long long)rows, (int)K, abs_max);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &row_abs_max_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(x),
+                       (long long)ldx, (long long)rows, (int)K, abs_max);
+  } else {
+    auto kf = &row_abs_max_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(x),
                        (long long)ldx, (long long)rows, (int)K, abs_max);
   }
   return launch_rc();
@@ -704,7 +736,7 @@ static ColSplit col_split(int dtype, int E, int K, int N) {
 
 int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* wmax,
                         void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
   if (!w || !wmax) return AMOE_ENULL;
   if (!aligned(w, esize(dtype)) || !aligned(wmax, 4)) return AMOE_EALIGN;
@@ -720,11 +752,14 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
     if (dtype == AMOE_F32) {
       auto kf = &weight_abs_max_kernel<float>;
       hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax, vec);
-    } else {
+    } else if (dtype == AMOE_BF16) {
       auto kf = &weight_abs_max_kernel<uint16_t>;
       hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax, vec);
+    } else {
+      auto kf = &weight_abs_max_kernel<f16_t>;
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const f16_t*>(w), per, wmax, vec);
     }
-  } else {
+  } else if (dtype == AMOE_BF16) {
     if ((long long)E * N > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(((long long)E * N + kThreads - 1) / kThreads)), dim3(kThreads), 0,
                        st, reinterpret_cast<uint32_t*>(wmax), (int)(E * N));
@@ -739,6 +774,23 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
     } else {
       auto kf = &weight_col_abs_max_kernel<uint16_t>;
       hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, width, wmax,
+                         vec);
+    }
+  } else {
+    if ((long long)E * N > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(((long long)E * N + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                       st, reinterpret_cast<uint32_t*>(wmax), (int)(E * N));
+    if (int rc = launch_rc()) return rc;
+    const ColSplit cs = col_split(dtype, E, K, N);
+    const int width = cs.width;
+    const int vec = aligned(w, 16) && (N % (16 / (int)esize(dtype)) == 0);
+    dim3 grid(cs.col_blocks, cs.slices, E);
+    if (dtype == AMOE_F32) {
+      auto kf = &weight_col_abs_max_kernel<float>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, width, wmax, vec);
+    } else {
+      auto kf = &weight_col_abs_max_kernel<f16_t>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const f16_t*>(w), (int)K, (int)N, width, wmax,
                          vec);
     }
   }
@@ -757,7 +809,7 @@ int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t 
 
 int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K, const int32_t* in_index,
                     const int32_t* offsets, int32_t E, float* out, void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (K < 1 || E < 1 || ldx < K) return AMOE_EINVAL;
   if (!x || !in_index || !offsets || !out) return AMOE_ENULL;
   if (!aligned(x, esize(dtype)) || !aligned(in_index, 4) || !aligned(offsets, 4) || !aligned(out, 4))
@@ -767,9 +819,13 @@ int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K, const 
     auto kf = &expert_std_kernel<float>;
     hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const float*>(x), (long long)ldx, (int)K,
                        in_index, offsets, out);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &expert_std_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(x), (long long)ldx, (int)K,
+                       in_index, offsets, out);
+  } else {
+    auto kf = &expert_std_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3(E), dim3(kThreads), 0, st, static_cast<const f16_t*>(x), (long long)ldx, (int)K,
                        in_index, offsets, out);
   }
   return launch_rc();
@@ -778,7 +834,7 @@ int amoe_expert_std(int32_t dtype, const void* x, int64_t ldx, int32_t K, const 
 int amoe_modify_weight(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, const float* wmax,
                        int32_t wmax_cols, float n_states, float std_dev, const float* noise, int32_t round_noise,
                        uint64_t noise_seed, const uint64_t* noise_seed_dev, void* out, void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (E < 1 || K < 1 || N < 1 || (wmax_cols != 1 && wmax_cols != N)) return AMOE_EINVAL;
   if (!w || !out || !wmax) return AMOE_ENULL;
   if (!aligned(w, esize(dtype)) || !aligned(out, esize(dtype)) || !aligned(wmax, 4) || !aligned(noise, 4) ||
@@ -798,8 +854,11 @@ int amoe_modify_weight(int32_t dtype, const void* w, int32_t E, int32_t K, int32
   if (dtype == AMOE_F32) {
     auto kf = &modify_weight_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, p);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &modify_weight_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, p);
+  } else {
+    auto kf = &modify_weight_kernel<f16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, p);
   }
   return launch_rc();
@@ -818,7 +877,7 @@ size_t amoe_weight_std_workspace(int32_t E, int32_t K, int32_t N, int32_t cols) 
 
 int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* std_out,
                     void* workspace, size_t workspace_bytes, void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
   if (!w || !std_out) return AMOE_ENULL;
   if (!aligned(w, esize(dtype)) || !aligned(std_out, 4) || !aligned(workspace, 8)) return AMOE_EALIGN;
@@ -837,9 +896,13 @@ int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t 
       auto kf = &weight_col_moments_kernel<float>;
       hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w), (int)K, (int)N, cs.width, partial,
                          vec);
-    } else {
+    } else if (dtype == AMOE_BF16) {
       auto kf = &weight_col_moments_kernel<uint16_t>;
       hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), (int)K, (int)N, cs.width,
+                         partial, vec);
+    } else {
+      auto kf = &weight_col_moments_kernel<f16_t>;
+      hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const f16_t*>(w), (int)K, (int)N, cs.width,
                          partial, vec);
     }
     if (int rc = launch_rc()) return rc;
@@ -853,9 +916,12 @@ int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t 
   if (dtype == AMOE_F32) {
     auto kf = &weight_moments_kernel<float>;
     hipLaunchKernelGGL(kf, dim3(slices, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, partial, vec);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &weight_moments_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3(slices, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, partial, vec);
+  } else {
+    auto kf = &weight_moments_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3(slices, E), dim3(kThreads), 0, st, static_cast<const f16_t*>(w), per, partial, vec);
   }
   if (int rc = launch_rc()) return rc;
   hipLaunchKernelGGL(weight_std_finalize_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st, partial,
@@ -865,7 +931,7 @@ int amoe_weight_std(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t 
 
 int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N, const float* bound, int32_t cols,
                        void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (E < 1 || K < 1 || N < 1 || (cols != 1 && cols != N)) return AMOE_EINVAL;
   if (!w || !bound) return AMOE_ENULL;
   if (!aligned(w, esize(dtype)) || !aligned(bound, 4)) return AMOE_EALIGN;
@@ -880,9 +946,13 @@ int amoe_clamp_weights(int32_t dtype, void* w, int32_t E, int32_t K, int32_t N, 
     auto kf = &clamp_weights_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<float*>(w), bound, rows, (int)K,
                        (int)N, (int)cols, vec, cvec);
-  } else {
+  } else if (dtype == AMOE_BF16) {
     auto kf = &clamp_weights_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<uint16_t*>(w), bound, rows,
+                       (int)K, (int)N, (int)cols, vec, cvec);
+  } else {
+    auto kf = &clamp_weights_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<f16_t*>(w), bound, rows,
                        (int)K, (int)N, (int)cols, vec, cvec);
   }
   return launch_rc();
@@ -898,7 +968,7 @@ size_t amoe_select_workspace(int64_t T, int32_t E) {
 
 int amoe_select_fwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k, void* sel_val, int64_t* sel_idx,
                     float* reg, float* reg_c, void* workspace, size_t workspace_bytes, void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || E < 1 || k < 1 || k > E) return AMOE_EINVAL;
   if (E > 64 * kSelPerLane) return AMOE_EUNSUPPORTED;
   if (T == 0) return AMOE_OK;
@@ -922,10 +992,14 @@ int amoe_select_fwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int
       auto kf = &select_fwd_kernel<float, PER>;                                                                        \
       hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(logits),         \
                          (long long)T, (int)E, (int)k, static_cast<float*>(sel_val), sel_idx, partial);                \
-    } else {                                                                                                           \
+    } else if (dtype == AMOE_BF16) {                                                                                   \
       auto kf = &select_fwd_kernel<uint16_t, PER>;                                                                     \
       hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(logits),      \
                          (long long)T, (int)E, (int)k, static_cast<uint16_t*>(sel_val), sel_idx, partial);             \
+    } else {                                                                                                           \
+      auto kf = &select_fwd_kernel<f16_t, PER>;                                                                        \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(logits),         \
+                         (long long)T, (int)E, (int)k, static_cast<f16_t*>(sel_val), sel_idx, partial);                \
     }                                                                                                                  \
   } while (0)
   if (E <= 64) AMOE_SELECT_FWD(1);
@@ -948,7 +1022,7 @@ int amoe_select_fwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int
 
 int amoe_select_bwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int32_t k, const int64_t* sel_idx,
                     const void* grad_val, const float* reg_c, const float* grad_reg, void* grad_logits, void* stream) {
-  if (dtype != AMOE_F32 && dtype != AMOE_BF16) return AMOE_EINVAL;
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || E < 1 || k < 1 || k > E) return AMOE_EINVAL;
   if (E > 64 * kSelPerLane) return AMOE_EUNSUPPORTED;
   if (T == 0) return AMOE_OK;
@@ -967,11 +1041,16 @@ int amoe_select_bwd(int32_t dtype, const void* logits, int64_t T, int32_t E, int
       hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(logits),         \
                          (long long)T, (int)E, (int)k, sel_idx, static_cast<const float*>(grad_val), reg_c, grad_reg,  \
                          static_cast<float*>(grad_logits));                                                            \
-    } else {                                                                                                           \
+    } else if (dtype == AMOE_BF16) {                                                                                   \
       auto kf = &select_bwd_kernel<uint16_t, PER>;                                                                     \
       hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(logits),      \
                          (long long)T, (int)E, (int)k, sel_idx, static_cast<const uint16_t*>(grad_val), reg_c,         \
                          grad_reg, static_cast<uint16_t*>(grad_logits));                                               \
+    } else {                                                                                                           \
+      auto kf = &select_bwd_kernel<f16_t, PER>;                                                                        \
+      hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(logits),         \
+                         (long long)T, (int)E, (int)k, sel_idx, static_cast<const f16_t*>(grad_val), reg_c,            \
+                         grad_reg, static_cast<f16_t*>(grad_logits));                                                  \
     }                                                                                                                  \
   } while (0)
   if (E <= 64) AMOE_SELECT_BWD(1);

@@ -23,6 +23,29 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   return (uint16_t)(pack_bf16x2(f, 0.f) & 0xffffu);   // hardware conversion, ties to even
 }
 
+// ---- fp16 <-> fp32 (round to nearest even) ----------------------------------------------------
+// The element type of fp16 tensors is f16_t; bf16 tensors are handled as their bits (uint16_t).
+typedef _Float16 f16_t;
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_v;
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_v;
+  const f32x2_v v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_v));
+}
+__device__ __forceinline__ void unpack_f16x2(uint32_t w, float& lo, float& hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_v;
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_v;
+  const f32x2_v v = __builtin_convertvector(__builtin_bit_cast(f16x2_v, w), f32x2_v);
+  lo = v[0];
+  hi = v[1];
+}
+template <typename T> constexpr bool kIsF16 = false;
+template <> constexpr bool kIsF16<f16_t> = true;
+// the 16 bits of one element, whatever its type
+template <typename T> __device__ __forceinline__ uint32_t elem_bits16(T v) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, v);
+}
+
 // Element traits.  Chunk = 16 bytes of elements, the unit of global and LDS vector access.
 template <typename T> struct Elem;
 template <> struct Elem<float> {
@@ -46,6 +69,19 @@ template <> struct Elem<uint16_t> {    // bf16 bits
   static __device__ __forceinline__ uint16_t cvt(float v) { return f32_to_bf16(v); }
   static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_to_f32(v); }
 };
+
+template <> struct Elem<f16_t> : Elem<uint16_t> {    // same tiling as bf16
+  static __device__ __forceinline__ float load(const f16_t* p) { return (float)*p; }
+  static __device__ __forceinline__ f16_t cvt(float v) { return (f16_t)v; }
+  static __device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
+};
+
+// 32 x 32 x 16 matrix instruction on 16-bit operands of type T
+template <typename T>
+__device__ __forceinline__ f32x16 mfma_32x32x16(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (kIsF16<T>) return mfma_32x32x16_f16(a, b, c);
+  else return mfma_32x32x16_bf16(a, b, c);
+}
 
 // ---- 16-byte chunks --------------------------------------------------------------------------
 // Operands travel global -> registers -> LDS as raw 16-byte chunks; only the gathered rows of
@@ -90,8 +126,8 @@ __device__ __forceinline__ Raw raw_load(const T* p, int n_valid, bool vec) {
   } else {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const uint32_t lo = (2 * j < n_valid) ? (uint32_t)p[2 * j] : 0u;
-      const uint32_t hi = (2 * j + 1 < n_valid) ? (uint32_t)p[2 * j + 1] : 0u;
+      const uint32_t lo = (2 * j < n_valid) ? elem_bits16(p[2 * j]) : 0u;
+      const uint32_t hi = (2 * j + 1 < n_valid) ? elem_bits16(p[2 * j + 1]) : 0u;
       r[j] = lo | (hi << 16);
     }
   }
@@ -112,6 +148,9 @@ __device__ __forceinline__ void raw_unpack(const Raw& r, float (&v)[Elem<T>::kCh
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
     for (int j = 0; j < 4; j++) v[j] = as_f32(r[j]);
+  } else if constexpr (kIsF16<T>) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) unpack_f16x2(r[j], v[2 * j], v[2 * j + 1]);
   } else {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -128,6 +167,9 @@ __device__ __forceinline__ Raw raw_pack(const float (&v)[Elem<T>::kChunk]) {
   if constexpr (sizeof(T) == 4) {
 #pragma unroll
     for (int j = 0; j < 4; j++) r[j] = as_u32(v[j]);
+  } else if constexpr (kIsF16<T>) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) r[j] = pack_f16x2(v[2 * j], v[2 * j + 1]);
   } else {
 #pragma unroll
     for (int j = 0; j < 4; j++) r[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
@@ -141,6 +183,12 @@ __device__ __forceinline__ Raw raw_pack_exact_bf16(const float (&v)[8]) {
 #pragma unroll
   for (int j = 0; j < 4; j++) r[j] = (as_u32(v[2 * j]) >> 16) | (as_u32(v[2 * j + 1]) & 0xffff0000u);
   return r;
+}
+// small integers (DAC codes) as 16-bit elements of T: exact in bf16 and in fp16
+template <typename T>
+__device__ __forceinline__ Raw raw_pack_codes(const float (&v)[8]) {
+  if constexpr (kIsF16<T>) return raw_pack<T>(v);
+  else return raw_pack_exact_bf16(v);
 }
 
 // a / b given y = 1/b (correctly rounded): one multiply and two fused multiply-adds give the
@@ -161,8 +209,8 @@ __device__ __forceinline__ void store4(T* p, const float (&v)[4], int n_valid, b
       *reinterpret_cast<f32x4*>(p) = o;
     } else {
       u32x2 o;
-      o[0] = pack_bf16x2(v[0], v[1]);
-      o[1] = pack_bf16x2(v[2], v[3]);
+      o[0] = kIsF16<T> ? pack_f16x2(v[0], v[1]) : pack_bf16x2(v[0], v[1]);
+      o[1] = kIsF16<T> ? pack_f16x2(v[2], v[3]) : pack_bf16x2(v[2], v[3]);
       *reinterpret_cast<u32x2*>(p) = o;
     }
   } else {
@@ -180,6 +228,10 @@ __device__ __forceinline__ void load4(const T* p, float (&v)[4], int n_valid, bo
       f32x4 o = *reinterpret_cast<const f32x4*>(p);
 #pragma unroll
       for (int j = 0; j < 4; j++) v[j] = o[j];
+    } else if constexpr (kIsF16<T>) {
+      u32x2 o = *reinterpret_cast<const u32x2*>(p);
+      unpack_f16x2(o[0], v[0], v[1]);
+      unpack_f16x2(o[1], v[2], v[3]);
     } else {
       u32x2 o = *reinterpret_cast<const u32x2*>(p);
       v[0] = as_f32(o[0] << 16);

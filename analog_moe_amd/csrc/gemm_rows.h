@@ -378,7 +378,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
               for (int j = 0; j < CH; j++) v[j] = dac_code_exact(xc[j], r, rinv, p.inp_res, inv_res);
             }
-            if constexpr (IS_BF16) ra[i] = raw_pack_exact_bf16(v);
+            if constexpr (IS_BF16) ra[i] = raw_pack_codes<T>(v);
             else ra[i] = raw_pack<T>(v);
           }
         }
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
               v[j] = x;
             }
             if (quant && out_of_range && a_ok[i] && p.range_flag != nullptr) atomicOr(p.range_flag, 1);
-            if constexpr (IS_BF16) a = codes_mode ? raw_pack_exact_bf16(v) : raw_pack<T>(v);
+            if constexpr (IS_BF16) a = codes_mode ? raw_pack_codes<T>(v) : raw_pack<T>(v);
             else a = raw_pack<T>(v);
           }
           *reinterpret_cast<Raw*>(&dA[((tid >> 3) + 32 * i) * LDA + a_chunk * CH]) = a;
@@ -449,7 +449,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
             for (int fi = 0; fi < 2; fi++)
 #pragma unroll
-              for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
+              for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16<T>(wf[fi], xf[ti], acc[fi][ti]);
           } else {
             float xf[2], wf[2];
 #pragma unroll
@@ -768,7 +768,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_rows_kernel(const RowsParams
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         float x = v[j];
-        if constexpr (IS_BF16) x = as_f32((uint32_t)Elem<T>::cvt(x) << 16);
+        if constexpr (IS_BF16) x = Elem<T>::to_f32(Elem<T>::cvt(x));
         xc[j] = clamp_sym(x, q_r);
         const float c = dac_code<IS_BF16>(xc[j], q_r, q_rinv, q_res, q_resinv, q_kq, tie);
         v[j] = IS_BF16 ? c : c * q_res;

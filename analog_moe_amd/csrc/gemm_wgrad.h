@@ -272,7 +272,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_wgrad_kernel(const WgradPara
 #pragma unroll
         for (int fn = 0; fn < 2; fn++)
 #pragma unroll
-          for (int fk = 0; fk < 2; fk++) acc[fn][fk] = mfma_32x32x16_bf16(gf[fn], xf[fk], acc[fn][fk]);
+          for (int fk = 0; fk < 2; fk++) acc[fn][fk] = mfma_32x32x16<T>(gf[fn], xf[fk], acc[fn][fk]);
       } else {
         float gf[2], xf[2];
 #pragma unroll

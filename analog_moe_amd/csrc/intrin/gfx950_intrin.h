@@ -26,6 +26,12 @@ __device__ __forceinline__ f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c)
                                                  __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// the same tile on fp16 operands (same operand layout)
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+__device__ __forceinline__ f32x16 mfma_32x32x16_f16(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
 // 32x32x32 signed 8-bit product, 32-bit integer accumulate: lane l supplies 16 bytes of row l%32 of each
 // operand (contraction indices 16*(l/32) .. +15); D as for the fp32 tiles.
 typedef __attribute__((ext_vector_type(16))) int i32x16;

@@ -84,8 +84,8 @@ class CVMM(torch.autograd.Function):
         E, K, N = keys.shape
         if torch.is_autocast_enabled():
             dt = torch.get_autocast_dtype("cuda")
-            if dt != torch.bfloat16:
-                raise RuntimeError("the CVMM kernels autocast to bfloat16 only")
+            if dt not in (torch.bfloat16, torch.float16):       # (the reference autocasts to float16: cvmm.py:716)
+                raise RuntimeError("the CVMM kernels autocast to bfloat16 or float16")
             x, keys_op = x.to(dt), keys.to(dt)
         else:
             keys_op = keys if keys.dtype == x.dtype else keys.to(x.dtype)

@@ -140,7 +140,7 @@ class SigmaMoELayer(nn.Module):
         return ((logits.is_cuda or logits.is_meta) and self.selection_mode == "sigmoid"
                 and not self.activation_after_topk and not (self.training and self.expert_dropout > 0)
                 and self.n_heads <= self.n_experts <= ops.SELECT_MAX_EXPERTS and logits.numel() > 0
-                and logits.dtype in (torch.float32, torch.bfloat16))
+                and logits.dtype in (torch.float32, torch.bfloat16, torch.float16))
 
     def _sel_activation(self, t: Tensor) -> Tensor:
         return torch.sigmoid(t) if self.selection_mode == "sigmoid" else F.softmax(t, dim=-1)
@@ -670,8 +670,8 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         lead = x.shape[:-1]
         if torch.is_autocast_enabled():            # as CVMM.forward does (cvmm.py:716): compute in the autocast type
             dt = torch.get_autocast_dtype("cuda")
-            if dt != torch.bfloat16:
-                raise MoEConifgError("the CVMM kernels autocast to bfloat16 only")
+            if dt not in (torch.bfloat16, torch.float16):
+                raise MoEConifgError("the CVMM kernels autocast to bfloat16 or float16")
             x = x.to(dt)
         y = moe_ffn(x.reshape(-1, x.shape[-1]), keys.to(x.dtype), values.to(x.dtype),
                     self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),

@@ -12,7 +12,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _abi
-from ._abi import AMOE_BF16, AMOE_F32, BwdWArgs, BwdXArgs, FwdArgs, check, set_bounds
+from ._abi import AMOE_BF16, AMOE_F16, AMOE_F32, BwdWArgs, BwdXArgs, FwdArgs, check, set_bounds
 
 
 def dtype_code(t: torch.Tensor) -> int:
@@ -20,7 +20,9 @@ def dtype_code(t: torch.Tensor) -> int:
         return AMOE_F32
     if t.dtype == torch.bfloat16:
         return AMOE_BF16
-    raise TypeError(f"unsupported dtype {t.dtype}: the CVMM kernels take float32 or bfloat16")
+    if t.dtype == torch.float16:
+        return AMOE_F16
+    raise TypeError(f"unsupported dtype {t.dtype}: the CVMM kernels take float32, bfloat16 or float16")
 
 
 def _p(t: Optional[torch.Tensor]):

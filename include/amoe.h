@@ -25,7 +25,7 @@ extern "C" {
 #define AMOE_VERSION 100
 #define AMOE_MAX_TILES 16   /* K-tiles per projection (max_input_size splitting) */
 
-enum { AMOE_F32 = 0, AMOE_BF16 = 1 };
+enum { AMOE_F32 = 0, AMOE_BF16 = 1, AMOE_F16 = 2 };
 
 enum {
   AMOE_OK = 0,
@@ -84,7 +84,7 @@ int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, in
  * extensions (the reference asserts them off: moe_layer_aihwkit_lightning.py:152-160).
  */
 typedef struct amoe_fwd_args {
-  int32_t dtype;                 /* AMOE_F32 / AMOE_BF16: type of x, w, out */
+  int32_t dtype;                 /* AMOE_F32 / AMOE_BF16 / AMOE_F16: type of x, w, out */
   int32_t M, N, K, E;            /* sorted rows, output features, input features, experts */
   int32_t n_in_rows, n_out_rows; /* rows of x / of out (indices are checked against nothing
                                     on the device; the caller guarantees the ranges).

@@ -46,11 +46,21 @@ def to_bf16(a: np.ndarray) -> np.ndarray:
     return out
 
 
+def to_f16(a: np.ndarray) -> np.ndarray:
+    """Round fp32 values to the nearest fp16 (ties to even, overflow to infinity); result kept in fp32."""
+    with np.errstate(over="ignore"):
+        return np.asarray(a, dtype=F32).astype(np.float16).astype(F32)
+
+
 def _cast(a: np.ndarray, dtype: str) -> np.ndarray:
+    """dtype "f32", "bf16" or "f16" (the reference's reduced-precision type, cvmm.py:177-179, 188-189): the values
+    as an element of that type holds them, kept in fp32."""
     if dtype == "f32":
         return np.asarray(a, dtype=F32)
     if dtype == "bf16":
         return to_bf16(a)
+    if dtype == "f16":
+        return to_f16(a)
     raise ValueError(dtype)
 
 
@@ -302,7 +312,7 @@ def cvmm_fwd(x, sel_index, sel_sorted, keys, inp_res=-1.0, ir=None, out_index=No
         wmax = np.asarray(wmax, dtype=F32).reshape(E, -1)
     out = np.zeros((M, N), dtype=F32)
     codes_all = np.zeros((M, K), dtype=F32) if return_codes else None
-    w_op = keys if dtype == "f32" else to_bf16(keys)
+    w_op = _cast(keys, dtype)
     for e in np.unique(sel_sorted):
         pos = np.nonzero(sel_sorted == e)[0]
         rin = sel_index[pos]
@@ -316,7 +326,7 @@ def cvmm_fwd(x, sel_index, sel_sorted, keys, inp_res=-1.0, ir=None, out_index=No
             if return_codes and codes is not None:
                 codes_all[pos, lo:hi] = codes
             if dtype != "f32" and codes is None:
-                a = to_bf16(a)
+                a = _cast(a, dtype)
             c = (a.astype(np.float64) @ w_op[e, lo:hi, :].astype(np.float64)).astype(F32)
             if noise is not None:
                 c = (c + noise[t, rout, :]).astype(F32)
@@ -385,7 +395,7 @@ def cvmm_bwd_w(x, sel_index, sel_sorted, grads, ir, n_experts, out_index=None, *
         pos = np.nonzero(sel_sorted == e)[0]
         a = _clip_rows(x[sel_index[pos]], None if ir is None else ir[pos], bounds)
         if dtype != "f32":
-            a = to_bf16(a)
+            a = _cast(a, dtype)
         out[e] = a.astype(np.float64).T @ grads[gidx[pos]].astype(np.float64)
     return _cast(out.astype(F32), dtype)
 
@@ -434,7 +444,7 @@ def cvmm_backward(grad_output, x, keys, sel_sorted, sel_index, out_index, gate, 
     # cvmm.py:828-846: plain gather-GEMM-scatter with W^T
     pos_out = sel_index if out_index is None else np.asarray(out_index).astype(np.int64)
     g_rows = pos_out // k if gate is not None else pos_out  # row of grad_output per sorted pos
-    w_op = keys if dtype == "f32" else to_bf16(keys)
+    w_op = _cast(keys, dtype)
     full = np.zeros((M, K), dtype=F32)                      # indexed by output row
     ir_grad = None if ir is None else np.zeros((M, nt), dtype=F32)
     xs = x[sel_index]                                       # sorted order (cvmm.py:851)

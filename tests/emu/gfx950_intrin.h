@@ -79,6 +79,29 @@ inline f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c) {
   return c;
 }
 
+inline f32x16 mfma_32x32x16_f16(u32x4 a, u32x4 b, f32x16 c) {
+  struct Ops { _Float16 a[8], b[8]; } mine;
+  std::memcpy(mine.a, &a, 16);
+  std::memcpy(mine.b, &b, 16);
+  EmuWave* w = emu_wave;
+  const int l = lane_id();
+  std::memcpy(w->slot[l], &mine, sizeof(mine));
+  w->bar.arrive_and_wait();
+  const int col = l % 32;
+  for (int i = 0; i < 16; i++) {
+    const int row = 8 * (i / 4) + 4 * (l / 32) + (i % 4);
+    float s = c[i];
+    for (int k = 0; k < 16; k++) {
+      const Ops* pa = (const Ops*)w->slot[row + 32 * (k / 8)];
+      const Ops* pb = (const Ops*)w->slot[col + 32 * (k / 8)];
+      s += (float)pa->a[k % 8] * (float)pb->b[k % 8];
+    }
+    c[i] = s;
+  }
+  w->bar.arrive_and_wait();
+  return c;
+}
+
 typedef __attribute__((ext_vector_type(16))) int i32x16;
 inline i32x16 mfma_i32_32x32x32_i8(u32x4 a, u32x4 b, i32x16 c) {
   struct Ops { int8_t a[16], b[16]; } mine;

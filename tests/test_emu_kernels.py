@@ -85,6 +85,16 @@ CASES = {
                       dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, bounds_up=[0, 96, 256]), "bf16", 2e-2),
     "f32_interior_ir_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(ir=True, decay=0.01), "f32", 1e-5),
     "f32_interior_quant_only": (dict(T=80, D=128, E=3, F=128, k=2), dict(inp_res=1 / 127), "f32", 1e-5),
+    # fp16, the reference's reduced-precision type (cvmm.py:177-179, 188-189): plain, ragged with the analog stages
+    # (per-position and per-expert ranges by turns), interior tiles
+    "f16_plain": (dict(T=48, D=128, E=4, F=64, k=2), dict(), "f16", 2e-3),
+    "f16_ragged_split_adc_noise": (dict(T=40, D=76, E=3, F=36, k=2),
+                                   dict(ir=True, inp_res=1 / 127, bounds_up=[0, 40, 76], out_bound=12.0, out_res=254.0,
+                                        noise=0.04, decay=0.01), "f16", 2e-3),
+    "f16_interior": (dict(T=80, D=128, E=3, F=128, k=2),
+                     dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01),
+                     "f16", 2e-3),
+    "f16_ir_quant": (dict(T=48, D=128, E=4, F=64, k=2), dict(ir=True, inp_res=1 / 127, decay=0.01), "f16", 2e-3),
 }
 
 
@@ -95,7 +105,7 @@ def test_layer_parity_emulated(emu_ops, name):
     # alternate between the per-position input-range vector of the reference and the fused
     # per-expert table / in-kernel gate (x) dy product
     lk["by_expert"] = list(CASES).index(name) % 2 == 1
-    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    tdt = util.TORCH_DTYPE[dtype]
     pr = util.make_problem(7, dtype=tdt, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
     ir = None

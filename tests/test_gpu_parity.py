@@ -1,6 +1,6 @@
 """GPU parity tests: the HIP kernels, called through the C ABI (analog_moe_amd.ops ->
 libamoe.so), against the CPU oracle on the same seeded inputs.
-Tolerances: selection bit-exact; fp32 1e-5 and bf16 2e-2 relative to the scale of the
+Tolerances: selection bit-exact; fp32 1e-5, bf16 2e-2 and fp16 2e-3 relative to the scale of the
 reference tensor (max |a-b| / max |b|)."""
 import numpy as np
 import pytest
@@ -11,7 +11,7 @@ from tests import util
 from tests.test_emu_kernels import CASES
 
 pytestmark = pytest.mark.gpu
-TOL = {"f32": 1e-5, "bf16": 2e-2}
+TOL = {"f32": 1e-5, "bf16": 2e-2, "f16": 2e-3}
 
 
 @pytest.fixture(scope="module")
@@ -47,7 +47,7 @@ def test_prepare_sel_bit_exact(ops, M, E, k, skew):
 
 def _run_case(ops, pk, lk, dtype, seed=7, routing="router", by_expert=False):
     lk = dict(lk, by_expert=by_expert)
-    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    tdt = util.TORCH_DTYPE[dtype]
     pr = util.make_problem(seed, dtype=tdt, routing=routing, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
     ir = None

@@ -30,6 +30,14 @@ def make_problem(seed, T, D, E, F, k, dtype=torch.float32, routing="router", dev
     return dict(x=cast(x), keys=cast(keys), values=cast(values), idx=idx.to(device), gate=cast(gate), dy=cast(dy))
 
 
+TORCH_DTYPE = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def dtype_name(dtype) -> str:
+    """The oracle's name of a torch dtype."""
+    return {v: n for n, v in TORCH_DTYPE.items()}[dtype]
+
+
 def np32(t):
     return None if t is None else t.detach().float().cpu().numpy()
 
@@ -174,7 +182,7 @@ def check_generated_noise_interior(ops, device="cpu", dtype=torch.bfloat16, spli
     per-expert input-range table: the straight-line output stage of the usual training configuration, with and
     without the K-tile split, against the oracle's counter noise.  Stage by stage: the oracle continues from
     the kernel's own first-stage output, and a value next to an ADC rounding boundary may differ by one step."""
-    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    name = dtype_name(dtype)
     pr = make_problem(23, T, D, E, F, k, dtype=dtype)
     bounds_up = [0, D // 2, D] if split else None
     nt = 2 if split else 1
@@ -286,7 +294,7 @@ def check_row_chunked_wgrad(ops, device="cpu", dtype=torch.float32, T=600, D=136
     tol = 1e-5 if dtype == torch.float32 else 2e-2
     want = O.cvmm_bwd_w(np32(x), in_index.cpu().numpy(), ss.cpu().numpy(), np32(g),
                         np.full((T * k, 1), 0.8, np.float32), E, perm.cpu().numpy(),
-                        dtype="f32" if dtype == torch.float32 else "bf16")
+                        dtype=dtype_name(dtype))
     outs = []
     for rows_per_chunk in (64, 64, 192, 1 << 20):
         got = ops.cvmm_bwd_w(x, g, E, offsets, in_index, perm, ir=ir, ir_by_expert=True,
@@ -364,7 +372,7 @@ def check_modify_weight(ops, kind, dtype=torch.float32, device="cpu", E=3, K=40,
                         seed=0x51EDC0DE12345):
     """The kernel against the oracle, bit for bit: once with injected normals, once with its own draws."""
     from oracle import weights_oracle as WO
-    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    name = dtype_name(dtype)
     w = modifier_weights(7, E, K, N, dtype, device)
     per_channel = kind in WO.PER_CHANNEL_WMAX
     wmax = ops.weight_abs_max(w, per_channel)
@@ -395,7 +403,7 @@ def check_modify_weight(ops, kind, dtype=torch.float32, device="cpu", E=3, K=40,
 
 def check_weight_clip(ops, per_channel, dtype=torch.float32, device="cpu", E=3, K=50, N=20, sigma=1.5):
     from oracle import weights_oracle as WO
-    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    name = dtype_name(dtype)
     w = (modifier_weights(9, E, K, N) + 0.5).to(dtype).to(device)       # a mean far from zero
     std = ops.weight_std(w, per_channel)
     want_std = WO.weight_std(np32(w), per_channel)
@@ -433,7 +441,7 @@ def check_select(ops, dtype=torch.float32, device="cpu", T=70, E=24, k=3, seed=0
     values; where gate values tie, the kernel takes the lower id like the oracle), regulariser and gradients to
     fp32 / bf16 accuracy."""
     from oracle import select_oracle as SO
-    name = "bf16" if dtype == torch.bfloat16 else "f32"
+    name = dtype_name(dtype)
     g = torch.Generator().manual_seed(seed)
     logits = (torch.randn(T, E, generator=g) * 2.0).to(dtype)
     logits[0, :] = logits[0, 0]                                     # a row of ties
