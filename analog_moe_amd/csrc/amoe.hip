@@ -98,35 +98,36 @@ int launch_rows(const RowsParams& p, int mode, int grid, hipStream_t st) {
                                             : launch_rows_mode<T, W_KC, false>(p, mode, grid, st);
 }
 
-// The 128 x 256 forward kernel for the usual training shapes (bf16, every tile interior, per-expert input
+// The 128 x 256 forward kernel for the usual training shapes (bf16 or fp16, every tile interior, per-expert input
 // ranges, one max |W| per expert).  AMOE_EUNSUPPORTED: this launch is not one of them; the general kernel runs.
-template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
+template <typename T, int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
 int launch_fwd256_as(const RowsParams& p, int grid, hipStream_t st) {
-  auto k = &fwd256_kernel<A_MODE, ANALOG, NOISE, SPLIT2, ZCODES>;
+  auto k = &fwd256_kernel<T, A_MODE, ANALOG, NOISE, SPLIT2, ZCODES>;
   hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), 0, st, p);
   return launch_rc();
 }
 
 // The 128 x 256 input-gradient kernel, for the same launches (and column tiles that are multiples of 256).  The
 // partial sums of the input-range gradient then cover 256 columns each; *n_count_blocks is the grid that ran.
-template <int COLS>
+template <typename T, int COLS>
 int launch_bwdx256_cols(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks) {
   p.n_col_blocks = count_col_blocks(p.col_bounds, p.n_col_tiles, COLS);
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks, COLS == 128 ? 3 : 2);
   *n_count_blocks = grid;
   const bool relu = a->relu_mask != 0, xc = a->xc_out != nullptr;
   if (a->x == nullptr) {
-    hipLaunchKernelGGL((&bwdx256_kernel<false, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    hipLaunchKernelGGL((&bwdx256_kernel<T, false, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
   } else if (!relu) {
-    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, false, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
-    else hipLaunchKernelGGL((&bwdx256_kernel<true, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<T, true, false, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<T, true, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
   } else {
-    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<true, true, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
-    else hipLaunchKernelGGL((&bwdx256_kernel<true, true, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    if (xc) hipLaunchKernelGGL((&bwdx256_kernel<T, true, true, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL((&bwdx256_kernel<T, true, true, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
   }
   return launch_rc();
 }
 
+template <typename T>
 int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks, int* block_cols) {
   if (!rows_all_interior(p, MODE_BWDX, kFBK)) return AMOE_EUNSUPPORTED;
   if (a->ir != nullptr && !a->ir_by_expert) return AMOE_EUNSUPPORTED;
@@ -134,9 +135,10 @@ int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* 
   for (int t = 0; t < a->n_tiles; t++)
     if ((a->tile_bounds[t + 1] - a->tile_bounds[t]) % kFCols) return AMOE_EUNSUPPORTED;
   *block_cols = kFCols;
-  return launch_bwdx256_cols<kFCols>(p, a, st, n_count_blocks);
+  return launch_bwdx256_cols<T, kFCols>(p, a, st, n_count_blocks);
 }
 
+template <typename T>
 int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st) {
   if (!rows_all_interior(p, mode, kFBK) || a->N % kFCols) return AMOE_EUNSUPPORTED;
   if (a->noise != nullptr || a->n_tiles > 2) return AMOE_EUNSUPPORTED;
@@ -149,29 +151,29 @@ int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st
   p.n_col_blocks = a->N / kFCols;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (a->code_out && !analog) return AMOE_EUNSUPPORTED;
-  if (!dac) return launch_fwd256_as<FA_PLAIN, false, false, false>(p, grid, st);
+  if (!dac) return launch_fwd256_as<T, FA_PLAIN, false, false, false>(p, grid, st);
   if (!analog)
-    return a->x_is_quantized ? launch_fwd256_as<FA_CODES, false, false, false>(p, grid, st)
-                             : launch_fwd256_as<FA_DAC, false, false, false>(p, grid, st);
+    return a->x_is_quantized ? launch_fwd256_as<T, FA_CODES, false, false, false>(p, grid, st)
+                             : launch_fwd256_as<T, FA_DAC, false, false, false>(p, grid, st);
   if (a->code_out) {
     // codes leave instead of values: one output quantiser whose half range fits a byte, no second output
     const float half = 0.5f * fmaxf(a->out_res, 1.0f / a->out_res);
     if (a->n_tiles != 1 || a->xq_out || a->relu || !(half <= 127.f) || !aligned(a->code_out, 16) || a->ldcode % 16)
       return AMOE_EUNSUPPORTED;
     if (a->x_is_quantized)
-      return noisy ? launch_fwd256_as<FA_CODES, true, true, false, true>(p, grid, st)
-                   : launch_fwd256_as<FA_CODES, true, false, false, true>(p, grid, st);
-    return noisy ? launch_fwd256_as<FA_DAC, true, true, false, true>(p, grid, st)
-                 : launch_fwd256_as<FA_DAC, true, false, false, true>(p, grid, st);
+      return noisy ? launch_fwd256_as<T, FA_CODES, true, true, false, true>(p, grid, st)
+                   : launch_fwd256_as<T, FA_CODES, true, false, false, true>(p, grid, st);
+    return noisy ? launch_fwd256_as<T, FA_DAC, true, true, false, true>(p, grid, st)
+                 : launch_fwd256_as<T, FA_DAC, true, false, false, true>(p, grid, st);
   }
   if (a->x_is_quantized)
-    return noisy ? launch_fwd256_as<FA_CODES, true, true, false>(p, grid, st)
-                 : launch_fwd256_as<FA_CODES, true, false, false>(p, grid, st);
+    return noisy ? launch_fwd256_as<T, FA_CODES, true, true, false>(p, grid, st)
+                 : launch_fwd256_as<T, FA_CODES, true, false, false>(p, grid, st);
   if (a->n_tiles == 2)
-    return noisy ? launch_fwd256_as<FA_DAC, true, true, true>(p, grid, st)
-                 : launch_fwd256_as<FA_DAC, true, false, true>(p, grid, st);
-  return noisy ? launch_fwd256_as<FA_DAC, true, true, false>(p, grid, st)
-               : launch_fwd256_as<FA_DAC, true, false, false>(p, grid, st);
+    return noisy ? launch_fwd256_as<T, FA_DAC, true, true, true>(p, grid, st)
+                 : launch_fwd256_as<T, FA_DAC, true, false, true>(p, grid, st);
+  return noisy ? launch_fwd256_as<T, FA_DAC, true, true, false>(p, grid, st)
+               : launch_fwd256_as<T, FA_DAC, true, false, false>(p, grid, st);
 }
 
 }  // namespace
@@ -356,8 +358,8 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
              ((long long)a->K * a->w_stride_k + (long long)a->N * a->w_stride_n) * (long long)es < lim;
   const int mode = a->n_tiles > 1 ? MODE_FWD_SPLIT : MODE_FWD;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (a->dtype == AMOE_BF16 && !w_kc) {
-    const int rc = launch_fwd256(p, mode, a, st);
+  if (a->dtype != AMOE_F32 && !w_kc) {
+    const int rc = a->dtype == AMOE_F16 ? launch_fwd256<f16_t>(p, mode, a, st) : launch_fwd256<uint16_t>(p, mode, a, st);
     if (rc != AMOE_EUNSUPPORTED) return rc;
   }
   if (a->code_out) return AMOE_EUNSUPPORTED;      // only the kernel above writes codes
@@ -537,9 +539,10 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   int block_cols = kTileCols, n_count_blocks = grid;
   int rc = AMOE_EUNSUPPORTED;
-  if (a->dtype == AMOE_BF16) {
+  if (a->dtype != AMOE_F32) {
     int cols = kTileCols;
-    rc = launch_bwdx256(p, a, st, &n_count_blocks, &cols);
+    rc = a->dtype == AMOE_F16 ? launch_bwdx256<f16_t>(p, a, st, &n_count_blocks, &cols)
+                              : launch_bwdx256<uint16_t>(p, a, st, &n_count_blocks, &cols);
     if (rc == AMOE_OK) block_cols = cols;
   }
   if (rc == AMOE_EUNSUPPORTED)

@@ -1,4 +1,4 @@
-// Input gradient of the CVMM path for the usual training shapes (bf16, every tile interior, one input range per
+// Input gradient of the CVMM path for the usual training shapes (bf16 or fp16, every tile interior, one input range per
 // expert and K-tile): the 128 x 256 counterpart of MODE_BWDX in gemm_rows.h, same arithmetic in the same order.
 //     G = g[g_index[i], :] @ W[e]^T                  (contraction over the forward's output features, which are
 //                                                      contiguous in W: both operands are staged k-contiguous)
@@ -16,9 +16,9 @@ namespace amoe {
 // MASKS: the forward input is read for the clip mask against the input range (infinite if there is none) and, with
 // RELU, for the ReLU mask.  XC: also leave gate * clamp(x, +-ir) at the rows of x (needs MASKS).  The optional gate
 // scales the result in every variant.
-template <bool MASKS, bool RELU, bool XC, int COLS = kFCols>
+template <typename T, bool MASKS, bool RELU, bool XC, int COLS = kFCols>
 __global__ __launch_bounds__(kThreads, COLS == 128 ? 3 : 2) void bwdx256_kernel(const RowsParams p) {
-  using T = uint16_t;
+  static_assert(sizeof(T) == 2, "16-bit elements: bf16 (as bits) or fp16");
   static_assert(COLS == 128 || COLS == 256, "output columns per workgroup tile");
   constexpr int BK = kFBK, CH = 8;
   constexpr int LDA = BK + 8, LDB = BK + 8;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kThreads, COLS == 128 ? 3 : 2) void bwdx256_kernel(
 #pragma unroll
       for (int fi = 0; fi < NB; fi++)
 #pragma unroll
-        for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
+        for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16<T>(wf[fi], xf[ti], acc[fi][ti]);
     };
     // the forward-input rows of one half of the tile: 64 rows x CPR pieces, 64 / RPP per thread (rows tid / CPR + RPP i)
     constexpr int NX = HALF_ROWS / RPP;

@@ -1,4 +1,4 @@
-// Forward row-gather GEMM of the CVMM path for the usual training shapes: bf16, every tile interior, one
+// Forward row-gather GEMM of the CVMM path for the usual training shapes: bf16 or fp16, every tile interior, one
 // input range per expert and K-tile, one max |W| per expert.  Same arithmetic, in the same order, as the
 // general kernel of gemm_rows.h (which keeps serving every other case); what differs is the shape of the work:
 //
@@ -28,9 +28,9 @@ enum { FA_PLAIN = 0, FA_DAC = 1, FA_CODES = 2 };   // what the gathered operand 
 // otherwise the accumulator leaves as it is (times inp_res * ir for code operands).  SPLIT2: exactly two K-tiles
 // (needs ANALOG).  ZCODES: the result leaves as its ADC codes + 128, one byte each (and the expert's step and input
 // range go to code_scale_out), instead of as values.
-template <int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
+template <typename T, int A_MODE, bool ANALOG, bool NOISE, bool SPLIT2, bool ZCODES = false>
 __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p) {
-  using T = uint16_t;
+  static_assert(sizeof(T) == 2, "16-bit elements: bf16 (as bits) or fp16");
   constexpr int BK = kFBK, CH = 8;
   constexpr int LDA = BK + 8;                       // 80-byte rows: 16 consecutive rows hit 16 disjoint bank groups
   constexpr int LDB = kFCols + 32;                  // 576-byte rows: the four rows of a transposing read are disjoint
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
 #pragma unroll
               for (int j = 0; j < CH; j++) v[j] = dac_code_exact(xc[j], ir_t, ir_inv, p.inp_res, inv_res);
             }
-            ra[i] = raw_pack_exact_bf16(v);
+            ra[i] = raw_pack_codes<T>(v);
           }
         }
       };
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
 #pragma unroll
         for (int fi = 0; fi < 4; fi++)
 #pragma unroll
-          for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16_bf16(wf[fi], xf[ti], acc[fi][ti]);
+          for (int ti = 0; ti < 2; ti++) acc[fi][ti] = mfma_32x32x16<T>(wf[fi], xf[ti], acc[fi][ti]);
       };
 
       load_step(0);
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
       float tie = 0.f, xc[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        const float x = as_f32((uint32_t)Elem<T>::cvt(v[j]) << 16);
+        const float x = Elem<T>::to_f32(Elem<T>::cvt(v[j]));
         xc[j] = clamp_sym(x, q_r);
         v[j] = dac_code<true>(xc[j], q_r, q_rinv, q_res, q_resinv, q_kq, tie);
       }

@@ -130,10 +130,10 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
 def codes_supported(x: torch.Tensor, w: torch.Tensor, *, ir_by_expert: bool, inp_res: float, n_tiles: int,
                     out_bound: float, out_res: float, noise: Optional[torch.Tensor], per_channel: bool) -> bool:
     """Whether ``cvmm_fwd(..., want_codes=True)`` has a kernel for this call: the 128 x 256 forward kernel
-    with an output quantiser of at most 254 states (bf16, every tile interior: N a multiple of 256, K of 32,
+    with an output quantiser of at most 254 states (bf16 or fp16, every tile interior: N a multiple of 256, K of 32,
     16-byte aligned rows; per-expert input ranges with input quantisation; one max |W| per expert; no injected
     noise; one K-tile).  A pure function of shapes and settings, so that traced code can rely on it."""
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not w.is_contiguous():
+    if x.dtype not in (torch.bfloat16, torch.float16) or w.dtype != x.dtype or not w.is_contiguous():
         return False
     E, K, N = w.shape
     x2_stride = x.stride(-2) if x.dim() >= 2 else K

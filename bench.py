@@ -5,7 +5,7 @@ expert sort -> up-projection (DAC, K-tile split, noise, ADC, ReLU) -> down-proje
 gate-weighted reduction, then the full backward (both weight gradients, both input gradients
 with clip masks, input-range gradients, gate gradient).  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c2|c2_f32|c4|c1]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c3_f16|c2|c2_f32|c4|c1|c5]
 
 The default workload is BASELINE.json's 64-expert tile-split layer (configs[2]), the one its
 metric's MFMA-peak target is quoted on.  Only one GPU is used; --gpus N > 1 exits.
@@ -29,6 +29,9 @@ CONFIGS = {
                    name="config2: d_model=412 E=16 F=128 k=4 8192 tokens fp32"),
     "c3": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="bf16", routing="uniform", mis=512, noise=0.04,
                name="config3: d_model=1024 (2x512 tiles) E=64 F=256 k=8 16384 tokens bf16 uniform routing"),
+    "c3_f16": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="f16", routing="uniform", mis=512, noise=0.04,
+                   name="config3 in fp16 (the reference's reduced-precision type): d_model=1024 (2x512 tiles) E=64 "
+                        "F=256 k=8 16384 tokens uniform routing"),
     "c4": dict(T=32768, D=2048, E=128, F=512, k=4, dtype="bf16", routing="zipf", mis=-1, noise=0.04,
                name="config4: d_model=2048 E=128 F=512 k=4 32768 tokens bf16 Zipf(1.2) routing"),
     # the layer inside its caller: a 16-layer decoder training step (attention and norms are stock PyTorch)
@@ -37,7 +40,7 @@ CONFIGS = {
                name="config5: 16-layer SigmaMoE decoder training step, d_model=1024, 16 heads, 64 experts x 256, "
                     "k=8, context 1024, batch 16, vocab 8000, bf16"),
 }
-PEAK = {"bf16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
+PEAK = {"bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}       # dense MFMA, MI355X
 # roofline.traffic (HBM bytes of the dominant launch) comes from profiles/bench_<config>_hbm_traffic.json, written by
 # bench_traffic.py from two rocprofv3 counter runs of this file; it is null when no such run is recorded or the
 # kernel sources changed after it.
@@ -228,7 +231,7 @@ def main():
         return bench_decoder(args, cfg)
     ops.get_lib()
     dev = torch.device("cuda:0")
-    tdt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[cfg["dtype"]]
     T, D, E, F, k = (cfg[n] for n in "TDEFk")
 
     rpu = cfgmod.TorchInferenceRPUConfig()

@@ -95,6 +95,11 @@ CASES = {
                      dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=254.0, noise=0.04, decay=0.01),
                      "f16", 2e-3),
     "f16_ir_quant": (dict(T=48, D=128, E=4, F=64, k=2), dict(ir=True, inp_res=1 / 127, decay=0.01), "f16", 2e-3),
+    # fp16 on the 128 x 256 kernels (per-expert ranges): plain, and two K-tiles with the analog stages
+    "f16_wide_plain": (dict(T=90, D=256, E=3, F=256, k=2), dict(), "f16", 2e-3),
+    "f16_wide_split": (dict(T=90, D=512, E=3, F=256, k=2),
+                       dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0, out_res=254.0,
+                            decay=0.01), "f16", 2e-3),
 }
 
 

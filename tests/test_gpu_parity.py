@@ -106,13 +106,14 @@ def test_config2_paper_scale_layer(ops, dtype):
     print(errs)
 
 
-def test_wide_tiles_layer(ops):
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_wide_tiles_layer(ops, dtype):
     """Several row tiles per expert and several work items per workgroup of the 128 x 256 kernels (forward and
     input gradient): two K-tiles of 256 columns, per-expert ranges, DAC / ADC, injected noise, range decay."""
-    print("wide tiles", flush=True)
+    print("wide tiles", dtype, flush=True)
     errs = _run_case(ops, dict(T=4096, D=512, E=8, F=256, k=2),
                      dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0, out_res=254.0,
-                          noise=0.04, decay=0.01, input_min_percentage=0.9), "bf16", seed=0, by_expert=True)
+                          noise=0.04, decay=0.01, input_min_percentage=0.9), dtype, seed=0, by_expert=True)
     print(errs)
 
 
@@ -136,7 +137,7 @@ def test_generated_noise_matches_counter_oracle(ops):
 
 
 @pytest.mark.parametrize("split", [False, True])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_generated_noise_interior(ops, dtype, split):
     """The output stage the benchmark times (edge-free tiles, bf16 codes, noise drawn in the kernel, ADC, one
     max |W| per expert, per-expert input ranges; with and without the K-tile split) against the oracle."""
@@ -149,10 +150,11 @@ def test_bf16_dac_codes_next_to_rounding_ties(ops):
     util.check_bf16_dac_codes_near_ties(ops, device="cuda", T=960)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("noisy", [False, True])
-def test_result_as_adc_codes(ops, noisy):
-    print("result as ADC codes", noisy, flush=True)
-    util.check_result_as_codes(ops, device="cuda", noisy=noisy, T=3000, D=1024, F=256, E=8, k=4)
+def test_result_as_adc_codes(ops, noisy, dtype):
+    print("result as ADC codes", noisy, dtype, flush=True)
+    util.check_result_as_codes(ops, device="cuda", noisy=noisy, T=3000, D=1024, F=256, E=8, k=4, dtype=dtype)
 
 
 def test_companions(ops):

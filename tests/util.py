@@ -194,7 +194,7 @@ def check_generated_noise_interior(ops, device="cpu", dtype=torch.bfloat16, spli
     okw = dict(lk, wmax_up=pr["keys"].float().abs().amax((1, 2)).reshape(E, 1).numpy(),
                wmax_down=pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy())
     want = layer_oracle(pr, ir, name, got=got, **okw)
-    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    tol = {torch.bfloat16: 2e-2, torch.float16: 2e-3, torch.float32: 1e-4}[dtype]
     errs = compare_layer(got, want, tol, adc_step=adc_steps(pr, ir, lk))
     # the noise is really there, and a different seed gives different noise
     clean = layer_ops_fwd_bwd(ops, dev, ir.to(device), by_expert=True, backward=False,
@@ -243,17 +243,17 @@ def check_bf16_dac_codes_near_ties(ops, device="cpu", T=96):
     np.testing.assert_array_equal(np32(img), codes2)
 
 
-def check_result_as_codes(ops, device="cpu", T=150, D=256, F=128, E=3, k=2, noisy=True):
+def check_result_as_codes(ops, device="cpu", T=150, D=256, F=128, E=3, k=2, noisy=True, dtype=torch.bfloat16):
     """A forward whose result leaves as ADC codes (one byte per value + two factors per expert): the values behind
-    the codes round to exactly the bf16 result of the ordinary call, and the gate reduction / gate gradient that
+    the codes round to exactly the 16-bit result of the ordinary call, and the gate reduction / gate gradient that
     read the codes agree with those that read the values."""
-    pr = make_problem(29, T, F, E, D, k, dtype=torch.bfloat16)          # (a down-projection: [M, F] -> [M, D])
+    pr = make_problem(29, T, F, E, D, k, dtype=dtype)                   # (a down-projection: [M, F] -> [M, D])
     M = T * k
     g = torch.Generator().manual_seed(2)
-    p1 = torch.relu(torch.randn(M, F, generator=g)).bfloat16().to(device)
-    values = (torch.randn(E, F, D, generator=g) / F ** 0.5).bfloat16().to(device)
+    p1 = torch.relu(torch.randn(M, F, generator=g)).to(dtype).to(device)
+    values = (torch.randn(E, F, D, generator=g) / F ** 0.5).to(dtype).to(device)
     idx, gate = pr["idx"].to(device), pr["gate"].to(device)
-    dy = torch.randn(T, D, generator=g).bfloat16().to(device)
+    dy = torch.randn(T, D, generator=g).to(dtype).to(device)
     ss, perm, in_index, offsets = ops.prepare_sel(idx, E, k)
     ir = torch.linspace(0.6, 1.4, E).reshape(E, 1).to(device)
     wmax = ops.weight_abs_max(values, False)
@@ -265,7 +265,7 @@ def check_result_as_codes(ops, device="cpu", T=150, D=256, F=128, E=3, k=2, nois
     codes, scale = ops.cvmm_fwd(p1, values, ss, offsets, perm, None, M, want_codes=True, **kw)
     assert codes.dtype == torch.uint8 and tuple(codes.shape) == (M, D) and tuple(scale.shape) == (E, 2)
     zf = ops.dequant_codes(codes, scale, idx)
-    assert torch.equal(zf.to(torch.bfloat16), z)
+    assert torch.equal(zf.to(dtype), z)
     c = codes.cpu().numpy().astype(np.int32) - 128
     assert np.abs(c).max() <= 127 and np.abs(c).max() > 20
     # gate reduction and gate gradient from the codes: against float64 on the exact values, and close to the
