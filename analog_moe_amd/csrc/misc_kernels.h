@@ -290,12 +290,24 @@ __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __res
   const long long hi = lo + span < per_expert ? lo + span : per_expert;
   constexpr int CH = Elem<T>::kChunk;
   float m = 0.f;
-  for (long long i = lo + (long long)tid * CH; i < hi; i += (long long)kThreads * CH) {
-    const int nv = hi - i < CH ? (int)(hi - i) : CH;
-    float v[CH];
-    raw_unpack<T>(raw_load<T>(base + i, nv, vec != 0), v);
+  // four pieces per thread in flight at a time (the weights are read once: what matters is the loads' latency)
+  constexpr int U = 4;
+  for (long long i0 = lo + (long long)tid * CH; i0 < hi; i0 += (long long)U * kThreads * CH) {
+    Raw r[U];
 #pragma unroll
-    for (int q = 0; q < CH; q++) m = fmaxf(m, fabsf(v[q]));
+    for (int u = 0; u < U; u++) {
+      const long long i = i0 + (long long)u * kThreads * CH;
+      const long long left = hi - i;
+      const int nv = left < 0 ? 0 : (left < CH ? (int)left : CH);
+      r[u] = raw_load<T>(base + (nv > 0 ? i : lo), nv, vec != 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      float v[CH];
+      raw_unpack<T>(r[u], v);
+#pragma unroll
+      for (int q = 0; q < CH; q++) m = fmaxf(m, fabsf(v[q]));
+    }
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, wave_shfl_xor(m, d));

@@ -257,11 +257,13 @@ def test_compiled_layer_equals_eager(fused):
         assert torch.equal(w, g)
 
 
-def test_reference_operator_matches_oracle():
+@pytest.mark.parametrize("out_dtype,name,tol", [(torch.float32, "f32", 1e-5), (torch.float16, "f16", 2e-3)])
+def test_reference_operator_matches_oracle(out_dtype, name, tol):
     """torch.ops.amoe.cvmm_quantized with the reference's calling convention (cvmm.py:531-631): a one-element
-    tensor of -1 stands for an absent argument."""
+    tensor of -1 stands for an absent argument; out_dtype float16 is what the reference passes under autocast
+    (cvmm.py:716)."""
     from analog_moe_amd.cvmm import cvmm_prepare_sel2
-    pr = util.make_problem(5, 96, 72, 5, 40, 2, dtype=torch.float32)
+    pr = util.make_problem(5, 96, 72, 5, 40, 2, dtype=out_dtype)
     pr = {n: t.cuda() for n, t in pr.items()}
     s = cvmm_prepare_sel2(pr["idx"].view(8, 12, 2), 5)
     minus = torch.tensor([-1.0], device="cuda")
@@ -270,14 +272,14 @@ def test_reference_operator_matches_oracle():
     noise = torch.randn(8, 12, 2, 40, device="cuda") * 0.01
     want_sel = O.prepare_sel(pr["idx"].cpu().numpy(), 5, 2)
     for ir_t, noise_t, inp_res in ((minus, minus, -1.0), (ir, minus, 1 / 127), (ir, noise, 1 / 127)):
-        out = torch.ops.amoe.cvmm_quantized(x, s.sel_index, s.sel, pr["keys"], ir_t, inp_res, torch.float32,
+        out = torch.ops.amoe.cvmm_quantized(x, s.sel_index, s.sel, pr["keys"], ir_t, inp_res, out_dtype,
                                             s.out_index, minus, noise_t)
-        assert out.shape == (8, 12, 2, 40)
+        assert out.shape == (8, 12, 2, 40) and out.dtype == out_dtype
         want = O.cvmm_fwd(util.np32(pr["x"]), want_sel.in_index, want_sel.sel_sorted, util.np32(pr["keys"]),
                           inp_res=inp_res, ir=None if ir_t is minus else util.np32(ir).reshape(-1, 1),
                           out_index=want_sel.perm,
-                          noise=None if noise_t is minus else util.np32(noise).reshape(1, -1, 40))
-        assert util.rel_err(util.np32(out).reshape(-1, 40), want) < 1e-5
+                          noise=None if noise_t is minus else util.np32(noise).reshape(1, -1, 40), dtype=name)
+        assert util.rel_err(util.np32(out).reshape(-1, 40), want) < tol
 
 
 def _aihwkit_layer(cfgmod, d=128, E=4, F=64, k=2, ir=True, **fw):
