@@ -1,11 +1,11 @@
 """HBM bytes per launch of the six GEMM launches of a bench.py step, from two rocprofv3 counter runs.
 
   cd /tmp; export TMPDIR=/tmp; cd <repository>
-  rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/prof/fetch -- python3 bench.py --steps 3 --warmup 1 \
+  rocprofv3 --pmc FETCH_SIZE --output-format csv -d prof_out/fetch -- python3 bench.py --steps 3 --warmup 1 \
       --no-cpu-baseline --no-graph --copy-calibration
-  rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/prof/write -- python3 bench.py --steps 3 --warmup 1 \
+  rocprofv3 --pmc WRITE_SIZE --output-format csv -d prof_out/write -- python3 bench.py --steps 3 --warmup 1 \
       --no-cpu-baseline --no-graph --copy-calibration
-  python3 bench_traffic.py gpurun_out/prof/fetch gpurun_out/prof/write --config c3
+  python3 bench_traffic.py prof_out/fetch prof_out/write --config c3
 
 writes profiles/bench_<config>_hbm_traffic.json (read by bench.py for roofline.traffic) and prints the table kept
 next to it as text.  Both counters are in KiB per dispatch; each is scaled by what it reads for the one 256 MiB
