@@ -156,6 +156,10 @@ def test_generated_noise_interior_bf16(emu_ops, split):
     util.check_generated_noise_interior(emu_ops, split=split, T=70)
 
 
+def test_wide_kernels_with_uneven_experts(emu_ops):
+    util.check_wide_kernels_uneven_experts(emu_ops)
+
+
 def test_bf16_dac_codes_next_to_rounding_ties(emu_ops):
     util.check_bf16_dac_codes_near_ties(emu_ops)
 

@@ -117,6 +117,12 @@ def test_wide_tiles_layer(ops, dtype):
     print(errs)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_wide_kernels_with_uneven_experts(ops, dtype):
+    print("wide kernels, uneven experts", dtype, flush=True)
+    print(util.check_wide_kernels_uneven_experts(ops, device="cuda", dtype=dtype, T=3000, E=9))
+
+
 def test_generated_noise_matches_counter_oracle(ops):
     pr = util.make_problem(9, T=500, D=256, E=8, F=128, k=2)
     ir = torch.full((2, 8, 1), 2.0)

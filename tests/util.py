@@ -205,6 +205,31 @@ def check_generated_noise_interior(ops, device="cpu", dtype=torch.bfloat16, spli
     return errs
 
 
+def check_wide_kernels_uneven_experts(ops, device="cpu", dtype=torch.bfloat16, T=150, D=256, F=256, E=5, k=2):
+    """The 128 x 256 kernels (per-expert ranges, DAC, ADC, range decay) when the experts' segments are as uneven as
+    they get: one expert without rows, one with more than a row tile, the rest with partly filled tiles."""
+    pr = make_problem(31, T, D, E, F, k, dtype=dtype)
+    idx = pr["idx"].clone()
+    idx[idx == E - 1] = 0                                # the last expert gets nothing, the first gets its share
+    idx[: max(T // 2, 140), 0] = 1                       # and expert 1 more than 128 rows
+    pr["idx"] = idx
+    counts = torch.bincount(idx.reshape(-1), minlength=E)
+    assert int(counts[E - 1]) == 0 and int(counts.max()) > 128
+    ir = torch.from_numpy(np.random.default_rng(5).uniform(0.9, 2.5, size=(2, E, 1)).astype(np.float32))
+    lk = dict(inp_res=1.0 / 127.0, out_bound=12.0, out_res=254.0, decay=0.01, input_min_percentage=0.5)
+    dev = {n: t.to(device) for n, t in pr.items()}
+    got = layer_ops_fwd_bwd(ops, dev, ir.to(device), by_expert=True, **lk)
+    okw = dict(lk, wmax_up=pr["keys"].float().abs().amax((1, 2)).reshape(E, 1).numpy(),
+               wmax_down=pr["values"].float().abs().amax((1, 2)).reshape(E, 1).numpy())
+    name = dtype_name(dtype)
+    want = layer_oracle(pr, ir, name, got=got, **okw)
+    tol = {torch.bfloat16: 2e-2, torch.float16: 2e-3}[dtype]
+    errs = compare_layer(got, want, tol, adc_step=adc_steps(pr, ir, lk))
+    # the expert without rows gets exact zeros as its weight gradients
+    assert float(got["grad_keys"][E - 1].abs().max()) == 0.0 and float(got["grad_values"][E - 1].abs().max()) == 0.0
+    return errs
+
+
 # (input range, bf16 input) pairs whose DAC code is one step off when the two divisions of cvmm.py:154, 163 are
 # replaced by one multiplication with (1 / range) * (1 / step): found by enumerating every bf16 value against
 # 40 000 random ranges (about one range in a thousand has such a value)
