@@ -6,6 +6,7 @@
 #include "gemm_rows.h"
 #include "gemm_fwd256.h"
 #include "gemm_bwdx256.h"
+#include "gemm_wgrad256.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
 #include "weight_kernels.h"
@@ -455,6 +456,27 @@ int amoe_cvmm_bwd_w(const amoe_bwd_w_args* a, void* stream) {
   if (grid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   const long long rgrid = (long long)a->E * p.n_k_blocks * p.n_n_blocks * kWgradReduceSplit;
   if (rgrid > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  // the 256 x 256 kernel for the training shapes (16-bit elements, interior tiles, per-expert ranges)
+  bool wide = a->dtype != AMOE_F32 && p.x_vec && p.g_vec && p.out_stage && p.buf_ok && a->N % kW256Tile == 0 &&
+              (a->ir == nullptr || a->ir_by_expert);
+  for (int t = 0; t < a->n_tiles && wide; t++) wide = (a->tile_bounds[t + 1] - a->tile_bounds[t]) % kW256Tile == 0;
+  if (wide) {
+    const long long grid256 = 8LL * ((pairs + 7) / 8) * (p.n_k_blocks / 2) * (p.n_n_blocks / 2);
+    if (a->dtype == AMOE_BF16) {
+      hipLaunchKernelGGL((&wgrad256_kernel<uint16_t>), dim3((unsigned)grid256), dim3(kW256Threads), 0, st, p);
+    } else {
+      hipLaunchKernelGGL((&wgrad256_kernel<f16_t>), dim3((unsigned)grid256), dim3(kW256Threads), 0, st, p);
+    }
+    if (int rc = launch_rc()) return rc;
+    if (p.rows_per_chunk > 0) {
+      if (a->dtype == AMOE_BF16) {
+        hipLaunchKernelGGL((&wgrad_reduce_kernel<uint16_t>), dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
+      } else {
+        hipLaunchKernelGGL((&wgrad_reduce_kernel<f16_t>), dim3((unsigned)rgrid), dim3(kThreads), 0, st, p);
+      }
+    }
+    return launch_rc();
+  }
   if (a->dtype == AMOE_F32) {
     auto k = &gemm_wgrad_kernel<float>;
     hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(kThreads), 0, st, p);

@@ -243,6 +243,11 @@ def test_row_chunked_weight_gradient(emu_ops, dtype):
     util.check_row_chunked_wgrad(emu_ops, dtype=dtype, T=200)
 
 
+def test_row_chunked_weight_gradient_wide_tiles(emu_ops):
+    """the 256 x 256 kernel: its partial tiles are laid out as the 128 x 128 tiles the second launch adds"""
+    util.check_row_chunked_wgrad(emu_ops, dtype=torch.bfloat16, T=200, D=512, F=256)
+
+
 @pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 128, 128, 60), (torch.bfloat16, 128, 128, 60),
                                          (torch.bfloat16, 72, 40, 60), (torch.bfloat16, 256, 256, 70)])
 def test_chained_projections(emu_ops, dtype, D, F, T):

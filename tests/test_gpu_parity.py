@@ -186,6 +186,12 @@ def test_row_chunked_weight_gradient(ops, dtype):
     util.check_row_chunked_wgrad(ops, device="cuda", dtype=dtype, T=4000)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_row_chunked_weight_gradient_wide_tiles(ops, dtype):
+    print("row-chunked weight gradient, 256 x 256 tiles", dtype, flush=True)
+    util.check_row_chunked_wgrad(ops, device="cuda", dtype=dtype, T=4000, D=512, F=256)
+
+
 @pytest.mark.parametrize("dtype,D,F,T", [(torch.float32, 256, 128, 700), (torch.bfloat16, 256, 128, 700),
                                          (torch.bfloat16, 72, 40, 700), (torch.float32, 100, 36, 700),
                                          (torch.bfloat16, 256, 256, 1000), (torch.bfloat16, 512, 256, 1000)])
