@@ -60,7 +60,7 @@ def family(kernel: str):
         return "fwd"
     if "bwdx256_kernel" in kernel:
         return "xgrad"
-    if "gemm_wgrad_kernel" in kernel:
+    if "gemm_wgrad_kernel" in kernel or "wgrad256_kernel" in kernel:
         return "wgrad"
     if "gemm_rows_kernel<" in kernel:            # <T, W_KC, MODE, FAST>: mode 2 is the input gradient
         args = kernel.split("gemm_rows_kernel<", 1)[1].split(">", 1)[0].split(",")

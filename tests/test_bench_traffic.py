@@ -9,6 +9,8 @@ def test_kernel_families():
     assert BT.family("void amoe::fwd256_kernel<unsigned short, 1, true, true, true, false>(amoe::RowsParams)") == "fwd"
     assert BT.family("void amoe::bwdx256_kernel<unsigned short, true, false, false, 128>(amoe::RowsParams)") == "xgrad"
     assert BT.family("void amoe::gemm_wgrad_kernel<unsigned short>(amoe::WgradParams)") == "wgrad"
+    assert BT.family("void amoe::wgrad256_kernel<unsigned short>(amoe::WgradParams)") == "wgrad"
+    assert BT.family("void amoe::wgrad_reduce_kernel<unsigned short>(amoe::WgradParams)") is None
     assert BT.family("void amoe::gemm_rows_kernel<float, true, 2, false>(amoe::RowsParams)") == "xgrad"
     assert BT.family("void amoe::gemm_rows_kernel<float, false, 1, false>(amoe::RowsParams)") == "fwd"
     assert BT.family("void amoe::head_reduce_kernel<unsigned short>(...)") is None
