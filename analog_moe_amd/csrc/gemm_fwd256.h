@@ -261,36 +261,45 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
                                (uint32_t)(c0 + wc * 128 + fi * 32) >> 5,
                                (uint32_t)(row0 + wr * 64 + ti * 32), lh);
             }
+            auto code_of = [&](int i) {       // the ADC code of accumulator element i of this block
+              float v = acc[fi][ti][i];
+              if (CODES) v *= p.inp_res;
+              if constexpr (NOISE) v = fmaf((float)zi[i], u_nzs, v);
+              v = clamp_sym(v, u_bound);
+              return rintf(v * u_q);
+            };
+            // (the tile test stays outside the element loops: inside them the compiler keeps one branch and one
+            // copy of the accumulator block per element)
+            if (SPLIT2 && t == 0) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-              uint32_t word = 0;
+              for (int q = 0; q < 4; q++) {
+                uint32_t word = 0;
 #pragma unroll
-              for (int j = 0; j < 4; j++) {
-                float v = acc[fi][ti][4 * q + j];
-                if (CODES) v *= p.inp_res;
-                if constexpr (NOISE) v = fmaf((float)zi[4 * q + j], u_nzs, v);
-                v = clamp_sym(v, u_bound);
-                const float code = rintf(v * u_q);
-                if constexpr (SPLIT2) {
-                  if (t == 0) {
-                    word = cvt_pk_u8_f32(code + 128.0f, j, word);
-                  } else {
-                    const float first = (float)((packed[fi][ti][q] >> (8 * j)) & 0xffu) - 128.0f;
-                    acc[fi][ti][4 * q + j] = (first * u_qinv) * ir_first + (code * u_qinv) * ir_t;
-                  }
-                } else if constexpr (ZCODES) {
-                  word = cvt_pk_u8_f32(code + 128.0f, j, word);
-                } else {
-                  acc[fi][ti][4 * q + j] = (code * u_qinv) * ir_t;
+                for (int j = 0; j < 4; j++) word = cvt_pk_u8_f32(code_of(4 * q + j) + 128.0f, j, word);
+                packed[SPLIT2 ? fi : 0][ti][q] = word;
+              }
+            } else if constexpr (SPLIT2) {
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                const uint32_t word = packed[fi][ti][q];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  const float first = (float)((word >> (8 * j)) & 0xffu) - 128.0f;
+                  acc[fi][ti][4 * q + j] = (first * u_qinv) * ir_first + (code_of(4 * q + j) * u_qinv) * ir_t;
                 }
               }
-              if constexpr (SPLIT2) {
-                if (t == 0) packed[fi][ti][q] = word;
-              }
-              if constexpr (ZCODES) {     // straight to the staged tile (the stage buffers are idle by now)
+            } else if constexpr (ZCODES) {  // straight to the staged tile (the stage buffers are idle by now)
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int j = 0; j < 4; j++) word = cvt_pk_u8_f32(code_of(4 * q + j) + 128.0f, j, word);
                 *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(sStage) + rl * (kFCols + 16) + wc * 128 +
                                              fi * 32 + 8 * q + 4 * lh) = word;
               }
+            } else {
+#pragma unroll
+              for (int i = 0; i < 16; i++) acc[fi][ti][i] = (code_of(i) * u_qinv) * ir_t;
             }
           }
         }
