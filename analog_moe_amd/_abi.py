@@ -60,6 +60,19 @@ class BwdXArgs(C.Structure):
     ]
 
 
+class KsumClipArgs(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32), ("T", C.c_int64), ("k", C.c_int32), ("D", C.c_int32), ("E", C.c_int32),
+        ("full", P), ("x", P), ("ldx", C.c_int64), ("sel", P), ("sel_is_i64", C.c_int32),
+        ("perm", P), ("offsets", P), ("ir", P),
+        ("n_tiles", C.c_int32), ("tile_bounds", C.c_int32 * (AMOE_MAX_TILES + 1)),
+        ("grad_x", P), ("ir_grad", P),
+        ("gradient_relative", C.c_int32), ("gradient_scale", C.c_float),
+        ("decay", C.c_float), ("input_min_percentage", C.c_float),
+        ("workspace", P), ("workspace_bytes", C.c_size_t),
+    ]
+
+
 I32, I64, F32, SZ = C.c_int32, C.c_int64, C.c_float, C.c_size_t
 
 PROTOTYPES = {
@@ -77,6 +90,8 @@ PROTOTYPES = {
     "amoe_cvmm_bwd_x": (C.c_int, [C.POINTER(BwdXArgs), P]),
     "amoe_gate_reduce": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
     "amoe_ksum": (C.c_int, [I32, P, P, I64, I32, I32, P]),
+    "amoe_ksum_clip_workspace": (SZ, [I64, I32, I32]),
+    "amoe_ksum_clip": (C.c_int, [C.POINTER(KsumClipArgs), P]),
     "amoe_gate_grad": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
     "amoe_gate_reduce_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),
     "amoe_gate_grad_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),

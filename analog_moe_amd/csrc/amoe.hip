@@ -634,6 +634,57 @@ int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, 
   return head_reduce(dtype, full, nullptr, out, T, k, D, stream);
 }
 
+constexpr int kHeadClipBlocks = 1024;      // workgroups of the head sum with the clip: four per CU, all resident
+
+size_t amoe_ksum_clip_workspace(int64_t T, int32_t k, int32_t n_tiles) {
+  if (T < 0 || k < 1 || n_tiles < 1) return 0;
+  return (size_t)n_tiles * (size_t)(T > 0 ? T * k : 1) * sizeof(float) + (size_t)kHeadClipBlocks * sizeof(int32_t);
+}
+
+int amoe_ksum_clip(const amoe_ksum_clip_args* a, void* stream) {
+  if (!a) return AMOE_ENULL;
+  if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16 && a->dtype != AMOE_F16) return AMOE_EINVAL;
+  if (a->T < 0 || a->k < 1 || a->D < 1 || a->E < 1 || a->E > kSelMaxExperts) return AMOE_EINVAL;
+  if (int rc = check_bounds(a->n_tiles, a->tile_bounds, a->D)) return rc;
+  const long long M = (long long)a->T * a->k;
+  if (M > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
+  if (a->T == 0) return AMOE_OK;
+  if (!a->full || !a->x || !a->sel || !a->perm || !a->offsets || !a->ir || !a->grad_x || !a->ir_grad || !a->workspace)
+    return AMOE_ENULL;
+  if (a->ldx < a->D) return AMOE_ESHAPE;
+  const int CH = a->dtype == AMOE_F32 ? 4 : 8;
+  if (!aligned(a->full, 16) || !aligned(a->x, 16) || !aligned(a->grad_x, 16) || !aligned(a->sel, a->sel_is_i64 ? 8 : 4) ||
+      !aligned(a->perm, 4) || !aligned(a->offsets, 4) || !aligned(a->ir, 4) || !aligned(a->ir_grad, 4) ||
+      !aligned(a->workspace, 4))
+    return AMOE_EALIGN;
+  if (a->k > 8 || a->D % CH || a->ldx % CH || !bounds_multiple_of(a->n_tiles, a->tile_bounds, CH)) return AMOE_EUNSUPPORTED;
+  if (a->workspace_bytes < amoe_ksum_clip_workspace(a->T, a->k, a->n_tiles)) return AMOE_EWORKSPACE;
+  HeadClipParams p{};
+  p.full = a->full; p.x = a->x; p.ldx = a->ldx; p.out = a->grad_x;
+  p.sel = a->sel; p.sel_is_i64 = a->sel_is_i64;
+  p.ir = a->ir; p.n_tiles = a->n_tiles;
+  for (int t = 0; t <= a->n_tiles; t++) p.bounds[t] = a->tile_bounds[t];
+  p.row_part = static_cast<float*>(a->workspace);
+  p.count = reinterpret_cast<int32_t*>(p.row_part + (size_t)a->n_tiles * M);
+  p.tokens = a->T; p.k = a->k; p.D = a->D;
+  const long long want = (a->T + 3) / 4;
+  const int blocks = (int)(want < kHeadClipBlocks ? want : kHeadClipBlocks);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a->dtype == AMOE_F32) hipLaunchKernelGGL((&head_sum_clip_kernel<float>), dim3(blocks), dim3(kThreads), 0, st, p);
+  else if (a->dtype == AMOE_BF16) hipLaunchKernelGGL((&head_sum_clip_kernel<uint16_t>), dim3(blocks), dim3(kThreads), 0, st, p);
+  else hipLaunchKernelGGL((&head_sum_clip_kernel<f16_t>), dim3(blocks), dim3(kThreads), 0, st, p);
+  if (int rc = launch_rc()) return rc;
+  IrFinalizeParams f{};
+  f.M = (int)M; f.n_tiles = a->n_tiles; f.KD_total = a->D; f.block_cols = a->D;     // one partial sum per K-tile
+  for (int t = 0; t <= a->n_tiles; t++) f.col_bounds[t] = a->tile_bounds[t];
+  f.irg_partial = p.row_part; f.notclip_count = p.count; f.n_blocks = blocks; f.row_index = a->perm;
+  f.ir = a->ir; f.ir_by_expert = 1; f.offsets = a->offsets; f.E = a->E; f.ir_grad = a->ir_grad;
+  f.relative = a->gradient_relative; f.scale = a->gradient_scale; f.decay = a->decay;
+  f.min_pct = a->input_min_percentage;
+  hipLaunchKernelGGL(ir_grad_finalize_kernel, dim3((unsigned)((M + kThreads - 1) / kThreads)), dim3(kThreads), 0, st, f);
+  return launch_rc();
+}
+
 int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D,
                    void* stream) {
   if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;

@@ -884,6 +884,7 @@ struct IrFinalizeParams {
   int block_cols;                // width of the column blocks the partial sums were made over
   int col_bounds[kMaxTiles + 1];
   const float* irg_partial; const int32_t* notclip_count; int n_blocks;
+  const int32_t* row_index;      // optional: the partial sums of sorted position r lie at row row_index[r]
   const float* ir; int ir_by_expert; const int32_t* offsets; int E; float* ir_grad;
   int relative; float scale, decay, min_pct;
 };
@@ -914,11 +915,12 @@ __global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFina
     }
     ir_row = lo;
   }
+  const int pr = p.row_index ? p.row_index[r] : r;
   int cb = 0;
   for (int t = 0; t < p.n_tiles; t++) {
     const int nb = (p.col_bounds[t + 1] - p.col_bounds[t] + p.block_cols - 1) / p.block_cols;
     float s = 0.f;
-    for (int b = 0; b < nb; b++) s += p.irg_partial[(int64_t)(cb + b) * p.M + r];
+    for (int b = 0; b < nb; b++) s += p.irg_partial[(int64_t)(cb + b) * p.M + pr];
     cb += nb;
     const float irv = p.ir[(int64_t)ir_row * p.n_tiles + t];
     if (p.relative) s = s * irv * p.scale;

@@ -217,6 +217,101 @@ __global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t
   }
 }
 
+// ---- the sum over the k heads of a per-head input gradient, with the input-range clip applied on the way -----
+// The clip mask of row r = t*k + j is |x[t, d]| < ir[e_r, tile(d)]: it depends on the token's input row, shared by
+// the k heads, and on one number per (expert, K-tile).  Applied here, the input row is read once per token instead
+// of once per head inside the GEMM that makes `full`, and that GEMM keeps no mask tile (cvmm.py:848-893, regrouped;
+// the reference masks the rounded product as well):
+//   out[t, d]        = sum_j [|x| < ir_j] full[t*k+j, d]                       fp32, ascending j
+//   row_part[tile][r] = sum_{d in tile} min([x >= ir] f, 0) - max([x <= -ir] f, 0)   lane's chunks in ascending d, then
+//                                                                                   over the lanes in a fixed order
+//   count[workgroup]  = number of (r, d) with |x| < ir
+// One wave per token (grid-stride); a lane owns 16-byte chunks; the k <= 8 head rows of a chunk are in flight together.
+// Tile bounds are multiples of the chunk.
+struct HeadClipParams {
+  const void* full; const void* x; long long ldx; void* out;
+  const void* sel; int sel_is_i64;
+  const float* ir; int n_tiles; int bounds[kMaxTiles + 1];
+  float* row_part; int32_t* count;
+  long long tokens; int k, D;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kThreads, 4) void head_sum_clip_kernel(const HeadClipParams p) {
+  constexpr int CH = Elem<T>::kChunk, JB = 8;
+  __shared__ int sCnt[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* __restrict__ FULL = static_cast<const T*>(p.full);
+  const T* __restrict__ X = static_cast<const T*>(p.x);
+  T* __restrict__ OUT = static_cast<T*>(p.out);
+  const int k = p.k, D = p.D;
+  const long long M = p.tokens * k;
+  int cnt = 0;
+  for (long long t = (long long)blockIdx.x * 4 + wave; t < p.tokens; t += (long long)gridDim.x * 4) {
+    int ej[JB];
+#pragma unroll
+    for (int jj = 0; jj < JB; jj++) ej[jj] = jj < k ? code_row_expert(p.sel, p.sel_is_i64, t * k + jj) : 0;
+    for (int tile = 0; tile < p.n_tiles; tile++) {
+      const int lo = p.bounds[tile], hi = p.bounds[tile + 1];
+      float irj[JB], part[JB];
+#pragma unroll
+      for (int jj = 0; jj < JB; jj++) {
+        irj[jj] = p.ir[(long long)ej[jj] * p.n_tiles + tile];
+        part[jj] = 0.f;
+      }
+      for (int d0 = lo; d0 < hi; d0 += 64 * CH) {      // (the same trip count in every lane: the vote below is wave-wide)
+        const int d = d0 + lane * CH;
+        const bool in = d < hi;
+        Raw rf[JB], rx = raw_zero();
+#pragma unroll
+        for (int jj = 0; jj < JB; jj++)
+          rf[jj] = (in && jj < k)
+                       ? __builtin_nontemporal_load(reinterpret_cast<const Raw*>(FULL + (t * k + jj) * (long long)D + d))
+                       : raw_zero();
+        if (in) rx = *reinterpret_cast<const Raw*>(X + t * p.ldx + d);
+        float xv[CH], acc[CH];
+        raw_unpack<T>(rx, xv);
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+          acc[q] = 0.f;
+          if (!in) xv[q] = __builtin_inff();   // a lane past the tile: clipped everywhere, and its zeros add nothing
+        }
+#pragma unroll
+        for (int jj = 0; jj < JB; jj++) {
+          if (jj < k) {
+            float v[CH];
+            raw_unpack<T>(rf[jj], v);
+#pragma unroll
+            for (int q = 0; q < CH; q++) {
+              const bool clipped = fabsf(xv[q]) >= irj[jj];
+              const float toward = as_f32(as_u32(v[q]) ^ (as_u32(xv[q]) & 0x80000000u));   // f * sign(x)
+              part[jj] += (clipped && toward < 0.f) ? toward : 0.f;                        // min([clipped] toward, 0)
+              cnt += popc64(wave_ballot(!clipped));                                          // (scalar unit; every lane votes)
+              acc[q] += clipped ? 0.f : v[q];
+            }
+          }
+        }
+        if (in) store_streaming(OUT + t * (long long)D + d, raw_pack<T>(acc));
+      }
+      // The eight row sums meet in ten exchanges instead of forty-eight: at distance 32 a lane hands over the four
+      // rows its partner keeps, at 16 two, at 8 one; three more steps finish the one row left, row lane / 8.
+      const bool b5 = (lane & 32) != 0, b4 = (lane & 16) != 0, b3 = (lane & 8) != 0;
+      float w4[4], w2[2];
+#pragma unroll
+      for (int i = 0; i < 4; i++) w4[i] = (b5 ? part[4 + i] : part[i]) + wave_shfl_xor(b5 ? part[i] : part[4 + i], 32);
+#pragma unroll
+      for (int i = 0; i < 2; i++) w2[i] = (b4 ? w4[2 + i] : w4[i]) + wave_shfl_xor(b4 ? w4[i] : w4[2 + i], 16);
+      float w1 = (b3 ? w2[1] : w2[0]) + wave_shfl_xor(b3 ? w2[0] : w2[1], 8);
+#pragma unroll
+      for (int s = 4; s >= 1; s >>= 1) w1 += wave_shfl_xor(w1, s);
+      if ((lane & 7) == 0 && (lane >> 3) < k) p.row_part[(long long)tile * M + t * k + (lane >> 3)] = w1;
+    }
+  }
+  if (lane == 0) sCnt[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) p.count[blockIdx.x] = sCnt[0] + sCnt[1] + sCnt[2] + sCnt[3];
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void row_abs_max_kernel(const T* __restrict__ x, long long ldx, long long rows,
                                                                 int K, float* __restrict__ out) {

@@ -143,8 +143,15 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
     gp1, irg_dn, p1c = ops.cvmm_bwd_x(dy, values, offsets, tok, perm, M, x=p1, xf_index=perm, gate=gate,
                                       ir=ir_dn, bounds=cfg.bounds_down, relu_mask=True, want_xc=True,
                                       **irkw, **by)
-    full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
-                                  bounds=cfg.bounds_up, **irkw, **by)
+    # the clip mask of the up-projection's input gradient depends on the token's input row, which its k heads
+    # share: where the sum over the heads can apply it, the GEMM runs without a mask tile and x is read once per
+    # token instead of once per head
+    late_clip = ir_up is not None and ops.ksum_clip_supported(x, k, cfg.bounds_up)
+    if late_clip:
+        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M)
+    else:
+        full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
+                                      bounds=cfg.bounds_up, **irkw, **by)
     # the gate gradient and the sum over the k heads only stream z, dy and the per-head input gradient
     # through HBM; they run on a second stream next to the two weight gradients, whose workgroups
     # leave registers and wave slots free on every CU
@@ -155,7 +162,11 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
             grad_gate = ops.gate_grad_codes(z, z_scale, sel_idx, dy, k).view(gate.shape)
         else:
             grad_gate = ops.gate_grad(z, dy, k).view(gate.shape)
-        grad_x = ops.ksum(full, k) if k > 1 else full
+        if late_clip:
+            grad_x, irg_up = ops.ksum_clip(full, x, sel_idx, perm, offsets, ir_up, k, bounds=cfg.bounds_up, **irkw)
+            irg_up.record_stream(main)
+        else:
+            grad_x = ops.ksum(full, k) if k > 1 else full
     grad_gate.record_stream(main)
     grad_x.record_stream(main)
     grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)

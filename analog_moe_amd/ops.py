@@ -242,6 +242,38 @@ def ksum(full: torch.Tensor, k: int) -> torch.Tensor:
     return out
 
 
+def ksum_clip_supported(x: torch.Tensor, k: int, bounds: Optional[Sequence[int]]) -> bool:
+    """Whether ``ksum_clip`` takes this case: 2 to 8 heads, rows of x and K-tile bounds on 16-byte chunks."""
+    ch = 4 if x.dtype == torch.float32 else 8
+    x2 = _rows2d(x)
+    b = [0, x2.shape[1]] if bounds is None else bounds
+    return (1 < k <= 8 and all(int(v) % ch == 0 for v in b) and x2.stride(0) % ch == 0
+            and x2.data_ptr() % 16 == 0)
+
+
+def ksum_clip(full: torch.Tensor, x: torch.Tensor, sel: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor,
+              ir: torch.Tensor, k: int, *, bounds: Optional[Sequence[int]] = None, gradient_relative: bool = True,
+              gradient_scale: float = 1.0, decay: float = 0.0, input_min_percentage: float = 0.95):
+    """``ksum`` of a per-head input gradient made without masks (``cvmm_bwd_x`` without x and ir), with the
+    input-range clip of x [T, D] against ir [E, n_tiles] applied on the way (cvmm.py:848-881, 890-891).
+    sel [..., k]: the expert of every (token, head).  Returns (grad_x [T, D], ir_grad [T*k, n_tiles] fp32 by
+    sorted position, as ``cvmm_bwd_x`` returns it)."""
+    _need_gpu(full, x, sel, perm, offsets, ir)
+    lib = get_lib()
+    f2 = _rows2d(full).contiguous()
+    x2 = _rows2d(x)
+    T, D = f2.shape[0] // k, f2.shape[1]
+    E = offsets.numel() - 1
+    ir32 = _f32c(ir)
+    n_tiles = 1 if bounds is None else len(bounds) - 1
+    grad_x = torch.empty((T, D), dtype=f2.dtype, device=f2.device)
+    ir_grad = torch.empty((T * k, n_tiles), dtype=torch.float32, device=f2.device)
+    ws = torch.empty(max(raw.ksum_clip_workspace_bytes(lib, T, k, n_tiles), 4), dtype=torch.uint8, device=f2.device)
+    raw.ksum_clip(lib, _stream(f2), f2, x2, sel.detach().reshape(-1).contiguous(), perm, offsets, ir32, grad_x, ir_grad,
+                  ws, T, k, E, bounds, gradient_relative, gradient_scale, decay, input_min_percentage)
+    return grad_x, ir_grad
+
+
 def gate_grad(z: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:
     _need_gpu(z, dy)
     z2, d2 = _rows2d(z).contiguous(), _rows2d(dy).contiguous()

@@ -12,7 +12,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _abi
-from ._abi import AMOE_BF16, AMOE_F16, AMOE_F32, BwdWArgs, BwdXArgs, FwdArgs, check, set_bounds
+from ._abi import AMOE_BF16, AMOE_F16, AMOE_F32, BwdWArgs, BwdXArgs, FwdArgs, KsumClipArgs, check, set_bounds
 
 
 def dtype_code(t: torch.Tensor) -> int:
@@ -218,6 +218,42 @@ def gate_grad_codes(lib, stream, codes, scale, sel, dy, grad_gate, T: int, k: in
 
 def ksum(lib, stream, full, out, T: int, k: int, D: int):
     check(lib, lib.amoe_ksum(dtype_code(full), _p(full), _p(out), T, k, D, stream), "amoe_ksum")
+
+
+def ksum_clip_workspace_bytes(lib, T: int, k: int, n_tiles: int) -> int:
+    return lib.amoe_ksum_clip_workspace(T, k, n_tiles)
+
+
+def ksum_clip(lib, stream, full, x, sel, perm, offsets, ir, grad_x, ir_grad, workspace, T: int, k: int, E: int,
+              bounds: Optional[Sequence[int]] = None, gradient_relative: bool = True, gradient_scale: float = 1.0,
+              decay: float = 0.0, input_min_percentage: float = 0.95):
+    """full [T*k, D] and grad_x [T, D] dense; x [T, D] rows; sel [T*k] int32 or int64; ir [E, n_tiles] fp32;
+    ir_grad [T*k, n_tiles] fp32 (by sorted position)."""
+    _rows(x, "x")
+    if not full.is_contiguous() or not grad_x.is_contiguous():
+        raise ValueError("full and grad_x must be contiguous")
+    if x.dtype != full.dtype or grad_x.dtype != full.dtype:
+        raise TypeError("full, x and grad_x share one dtype")
+    if sel.dtype not in (torch.int32, torch.int64) or not sel.is_contiguous() or sel.numel() != T * k:
+        raise TypeError("sel must be a contiguous int32 or int64 tensor of T * k experts")
+    D = full.shape[1]
+    if full.shape[0] != T * k or x.shape != (T, D) or grad_x.shape != (T, D):
+        raise ValueError("full / x / grad_x shapes do not match")
+    a = KsumClipArgs()
+    a.dtype = dtype_code(full)
+    a.T, a.k, a.D, a.E = T, k, D, E
+    a.full, a.x, a.ldx = _p(full), _p(x), x.stride(0)
+    a.sel, a.sel_is_i64 = _p(sel), int(sel.dtype == torch.int64)
+    a.perm, a.offsets = _p(_i32(perm, "perm")), _p(_i32(offsets, "offsets"))
+    a.ir = _p(_f32(ir, "ir"))
+    set_bounds(a, [0, D] if bounds is None else bounds)
+    if ir.numel() != E * a.n_tiles:
+        raise ValueError("ir must be [E, n_tiles]")
+    a.grad_x, a.ir_grad = _p(grad_x), _p(_f32(ir_grad, "ir_grad"))
+    a.gradient_relative, a.gradient_scale = int(bool(gradient_relative)), float(gradient_scale)
+    a.decay, a.input_min_percentage = float(decay), float(input_min_percentage)
+    a.workspace, a.workspace_bytes = _p(workspace), workspace.numel() * workspace.element_size()
+    check(lib, lib.amoe_ksum_clip(C.byref(a), stream), "amoe_ksum_clip")
 
 
 def gate_grad(lib, stream, z, dy, grad_gate, T: int, k: int, D: int):

@@ -238,6 +238,37 @@ int amoe_gate_reduce(int32_t dtype, const void* z, const void* gate, void* y,
 /* out[t, :] = sum_j full[t*k + j, :]           (cvmm.py:890-891) */
 int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, int32_t D,
               void* stream);
+/* amoe_ksum with the input-range clip of the up-projection applied on the way (cvmm.py:848-881 and 890-891,
+ * regrouped).  The clip mask of row r = t*k + j is |x[t, :]| < ir[sel[r], tile]: it depends on the token's input
+ * row, shared by its k heads, so the GEMM that makes `full` (amoe_cvmm_bwd_x without x and ir) keeps no mask tile
+ * and the input row is read once per token:
+ *   grad_x[t, :]  = sum_j [|x[t]| < ir] full[t*k + j, :]                                   (:853, 881, 890-891)
+ *   ir_grad[i, t] = sum_n min([x >= ir] full, 0) - sum_n max([x <= -ir] full, 0), row perm[i]  (:863-865)
+ *   then the scaling and decay rules of amoe_cvmm_bwd_x                                      (:868-878)
+ * full [T*k, D] and grad_x [T, D] are dense; x is [T, D] with row stride ldx; sel [T*k] holds the expert of
+ * every row (the unsorted ids, int32 or int64); perm [T*k] and offsets [E+1] are amoe_prepare_sel's; ir is
+ * [E, n_tiles].  ir_grad [T*k, n_tiles] is indexed by sorted position like amoe_cvmm_bwd_x's.
+ * k <= 8, tile bounds multiples of 16 bytes of elements; otherwise AMOE_EUNSUPPORTED (use amoe_cvmm_bwd_x with
+ * x and ir, then amoe_ksum).  workspace: amoe_ksum_clip_workspace(T, k, n_tiles) bytes. */
+typedef struct amoe_ksum_clip_args {
+  int32_t dtype;
+  int64_t T;  int32_t k, D, E;
+  const void* full;
+  const void* x;  int64_t ldx;
+  const void* sel;  int32_t sel_is_i64;
+  const int32_t* perm;  const int32_t* offsets;
+  const float* ir;
+  int32_t n_tiles;
+  int32_t tile_bounds[AMOE_MAX_TILES + 1];
+  void* grad_x;
+  float* ir_grad;
+  int32_t gradient_relative;  float gradient_scale;
+  float decay;  float input_min_percentage;
+  void* workspace;  size_t workspace_bytes;
+} amoe_ksum_clip_args;
+
+size_t amoe_ksum_clip_workspace(int64_t T, int32_t k, int32_t n_tiles);
+int amoe_ksum_clip(const amoe_ksum_clip_args* args, void* stream);
 /* grad_gate[t*k + j] = <z[t*k + j, :], dy[t, :]>   (cvmm.py:889) */
 int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate,
                    int64_t T, int32_t k, int32_t D, void* stream);

@@ -183,6 +183,26 @@ def test_companions(emu_ops):
     assert not (std[4] > 0)
 
 
+@pytest.mark.parametrize("dtype,kw", [
+    (torch.float32, dict(T=50, D=96, k=3, bounds=[0, 32, 96])),
+    (torch.float32, dict(T=9, D=260, k=2, E=2, strided_x=True, decay=0.0)),
+    (torch.bfloat16, dict(T=40, D=1040, k=8, E=9, bounds=[0, 520, 1040], sel_dtype=torch.int32)),
+    (torch.float16, dict(T=33, D=136, k=4, strided_x=True, input_min_percentage=0.99)),
+])
+def test_head_sum_with_input_range_clip(emu_ops, dtype, kw):
+    util.check_ksum_clip(emu_ops, dtype=dtype, **kw)
+
+
+def test_head_sum_with_clip_rejects_what_it_does_not_take(emu_ops):
+    x = torch.randn(4, 64)
+    assert not emu_ops.ksum_clip_supported(x, 1, None) and not emu_ops.ksum_clip_supported(x, 9, None)
+    assert not emu_ops.ksum_clip_supported(x, 2, [0, 30, 64]) and emu_ops.ksum_clip_supported(x, 2, [0, 32, 64])
+    idx = torch.zeros(4, 9, dtype=torch.int64)
+    s = emu_ops.prepare_sel(idx, 1, 9)
+    with pytest.raises(RuntimeError, match="not supported"):
+        emu_ops.ksum_clip(torch.randn(36, 64), x, idx, s[1], s[3], torch.ones(1, 1), 9)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", util.MODIFIER_KINDS)
 def test_weight_modifier_matches_oracle(emu_ops, kind, dtype):

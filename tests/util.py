@@ -95,6 +95,17 @@ def layer_ops_fwd_bwd(ops, pr, ir=None, *, inp_res=-1.0, noise_up=None, noise_do
     full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
                                   bounds=bounds_up, **irkw, **be)
     res["grad_x"] = ops.ksum(full, k)
+    if by_expert and ir is not None and ops.ksum_clip_supported(x, k, bounds_up):
+        # the same two results with the clip applied by the sum over the heads (the fused layer's order): the
+        # input gradient must not change by a bit; the input-range sums go on to the oracle comparison
+        plain, none = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M)
+        assert none is None
+        late_x, late_irg = ops.ksum_clip(plain, x, idx, perm, offsets, ir_up, k, bounds=bounds_up, **irkw)
+        assert torch.equal(late_x, res["grad_x"])
+        scale = float(irg_up.abs().max()) + 1e-30
+        assert float((late_irg - irg_up).abs().max()) / scale < (1e-5 if x.dtype == torch.float32 else 2e-2)
+        irg_up = late_irg
+        res["late_clip"] = True
     res["grad_p1"] = gp1
     if ir is not None:
         nt = ir.shape[2]
@@ -382,6 +393,37 @@ def check_clipped_input_output(ops, device="cpu", dtype=torch.float32, T=100, D=
 # ---------------------------------------------------------------------------------- weight modifier / clip
 MODIFIER_KINDS = ("DISCRETIZE", "DISCRETIZE_PER_CHANNEL", "ADD_NORMAL", "ADD_NORMAL_PER_CHANNEL",
                   "DISCRETIZE_ADD_NORMAL", "DISCRETIZE_ADD_NORMAL_PER_CHANNEL")
+
+
+def check_ksum_clip(ops, device="cpu", dtype=torch.float32, T=50, D=96, N=40, E=5, k=3, bounds=None, sel_dtype=torch.int64,
+                    strided_x=False, decay=0.01, input_min_percentage=0.5):
+    """The up-projection's input gradient as the fused layer makes it (plain GEMM, then the sum over the heads
+    with the clip) against the oracle's CVMM.backward and, bit for bit, against the masked GEMM followed by ksum."""
+    g = torch.Generator().manual_seed(T + D + k)
+    x = torch.randn(T, D + (8 if strided_x else 0), generator=g).to(dtype).to(device)[:, :D]
+    keys = (torch.randn(E, D, N, generator=g) / N ** 0.5).to(dtype).to(device)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(sel_dtype).to(device)
+    grads = torch.randn(T * k, N, generator=g).to(dtype).to(device)
+    nt = 1 if bounds is None else len(bounds) - 1
+    ir = torch.from_numpy(np.random.default_rng(5).uniform(0.4, 1.6, size=(E, nt)).astype(np.float32)).to(device)
+    sel_sorted, perm, in_index, offsets = ops.prepare_sel(idx, E, k)
+    M = T * k
+    kw = dict(gradient_relative=True, gradient_scale=0.7, decay=decay, input_min_percentage=input_min_percentage)
+    assert ops.ksum_clip_supported(x, k, bounds)
+    plain, _ = ops.cvmm_bwd_x(grads, keys, offsets, perm, perm, M)
+    got_x, got_irg = ops.ksum_clip(plain, x, idx, perm, offsets, ir, k, bounds=bounds, **kw)
+    masked, irg2 = ops.cvmm_bwd_x(grads, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir, bounds=bounds,
+                                  ir_by_expert=True, **kw)
+    assert torch.equal(got_x, ops.ksum(masked, k))
+    name = dtype_name(dtype)
+    want = O.cvmm_backward(np32(grads), np32(x), np32(keys), sel_sorted.cpu().numpy(), in_index.cpu().numpy(),
+                           perm.cpu().numpy(), None, ir[sel_sorted.long()].cpu().numpy(), None, k=k, bounds=bounds,
+                           dtype=name, **kw)
+    tol = {"f32": 1e-5, "bf16": 2e-2, "f16": 2e-3}[name]
+    assert rel_err(np32(got_x), want.grad_x) < tol
+    assert rel_err(got_irg.cpu().numpy(), want.ir_grad) < tol
+    clipped = (x.float().abs()[:, None, :] >= 0.4).float().mean()
+    assert 0.05 < float(clipped) < 0.95          # both sides of the mask occur
 
 
 def modifier_weights(seed, E, K, N, dtype=torch.float32, device="cpu"):
