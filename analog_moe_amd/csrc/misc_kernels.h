@@ -37,9 +37,25 @@ __global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restri
   }
 }
 
+// Wave sums of eight per-lane values in ten exchanges instead of forty-eight: at distance 32 a lane hands over the
+// four values its partner keeps, at 16 two, at 8 one; three more steps finish the one left.  Returns the sum of
+// v[lane / 8] (the same in the eight lanes of a group); fixed order.
+__device__ __forceinline__ float wave_sum8(const float (&v)[8], int lane) {
+  const bool b5 = (lane & 32) != 0, b4 = (lane & 16) != 0, b3 = (lane & 8) != 0;
+  float w4[4], w2[2];
+#pragma unroll
+  for (int i = 0; i < 4; i++) w4[i] = (b5 ? v[4 + i] : v[i]) + wave_shfl_xor(b5 ? v[i] : v[4 + i], 32);
+#pragma unroll
+  for (int i = 0; i < 2; i++) w2[i] = (b4 ? w4[2 + i] : w4[i]) + wave_shfl_xor(b4 ? w4[i] : w4[2 + i], 16);
+  float w1 = (b3 ? w2[1] : w2[0]) + wave_shfl_xor(b3 ? w2[0] : w2[1], 8);
+#pragma unroll
+  for (int s = 4; s >= 1; s >>= 1) w1 += wave_shfl_xor(w1, s);
+  return w1;
+}
+
 // grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>.  One wave per token: a lane's chunk of dy[t] is loaded once and
 // meets the same chunk of up to 8 head rows, whose loads are all in flight together.  Per row the sum runs
-// over the lane's chunks in ascending order, then over the lanes by a butterfly: independent of k.
+// over the lane's chunks in ascending order, then over the lanes in a fixed order: independent of k.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict__ z, const T* __restrict__ dy,
                                                               T* __restrict__ out, long long tokens, int k, int D,
@@ -69,13 +85,8 @@ __global__ __launch_bounds__(kThreads) void gate_grad_kernel(const T* __restrict
         for (int q = 0; q < CH; q++) s[jj] += a[q] * b[q];
       }
     }
-#pragma unroll
-    for (int jj = 0; jj < JB; jj++) {
-      float v = s[jj];
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) v += wave_shfl_xor(v, d);
-      if (lane == 0 && j0 + jj < k) out[t * k + j0 + jj] = Elem<T>::cvt(v);
-    }
+    const float v = wave_sum8(s, lane);
+    if ((lane & 7) == 0 && j0 + (lane >> 3) < k) out[t * k + j0 + (lane >> 3)] = Elem<T>::cvt(v);
   }
 }
 
@@ -199,19 +210,15 @@ __global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t
     }
 #pragma unroll
     for (int u = 0; u < TK; u++) {
-      float vb = sb[u];
+      // the offset leaves before the lanes meet (128 * sum dy is exact in every lane), then eight sums in one pass
 #pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) vb += wave_shfl_xor(vb, d);
-#pragma unroll
-      for (int jj = 0; jj < JB; jj++) {
-        float v = s[u][jj];
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) v += wave_shfl_xor(v, d);
-        if (lane == 0 && j0 + jj < k && t0 + u < tokens) {
-          const long long r = (t0 + u) * k + j0 + jj;
-          const int e = code_row_expert(sel, sel_is_i64, r);
-          out[r] = Elem<T>::cvt(((v - 128.0f * vb) * scale[2 * e]) * scale[2 * e + 1]);
-        }
+      for (int jj = 0; jj < JB; jj++) s[u][jj] -= 128.0f * sb[u];
+      const float v = wave_sum8(s[u], lane);
+      const int jj = lane >> 3;
+      if ((lane & 7) == 0 && j0 + jj < k && t0 + u < tokens) {
+        const long long r = (t0 + u) * k + j0 + jj;
+        const int e = code_row_expert(sel, sel_is_i64, r);
+        out[r] = Elem<T>::cvt((v * scale[2 * e]) * scale[2 * e + 1]);
       }
     }
   }
@@ -293,17 +300,7 @@ __global__ __launch_bounds__(kThreads, 4) void head_sum_clip_kernel(const HeadCl
         }
         if (in) store_streaming(OUT + t * (long long)D + d, raw_pack<T>(acc));
       }
-      // The eight row sums meet in ten exchanges instead of forty-eight: at distance 32 a lane hands over the four
-      // rows its partner keeps, at 16 two, at 8 one; three more steps finish the one row left, row lane / 8.
-      const bool b5 = (lane & 32) != 0, b4 = (lane & 16) != 0, b3 = (lane & 8) != 0;
-      float w4[4], w2[2];
-#pragma unroll
-      for (int i = 0; i < 4; i++) w4[i] = (b5 ? part[4 + i] : part[i]) + wave_shfl_xor(b5 ? part[i] : part[4 + i], 32);
-#pragma unroll
-      for (int i = 0; i < 2; i++) w2[i] = (b4 ? w4[2 + i] : w4[i]) + wave_shfl_xor(b4 ? w4[i] : w4[2 + i], 16);
-      float w1 = (b3 ? w2[1] : w2[0]) + wave_shfl_xor(b3 ? w2[0] : w2[1], 8);
-#pragma unroll
-      for (int s = 4; s >= 1; s >>= 1) w1 += wave_shfl_xor(w1, s);
+      const float w1 = wave_sum8(part, lane);          // row lane / 8
       if ((lane & 7) == 0 && (lane >> 3) < k) p.row_part[(long long)tile * M + t * k + (lane >> 3)] = w1;
     }
   }
