@@ -308,7 +308,7 @@ def main():
     # pass 1 (eager): HIP events around every launch give the per-launch durations
     saved = {}
     for name in ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x", "prepare_sel", "gate_reduce", "gate_grad", "ksum",
-                 "weight_abs_max", "segment_sum", "gate_reduce_codes", "gate_grad_codes"):
+                 "ksum_clip", "weight_abs_max", "segment_sum", "gate_reduce_codes", "gate_grad_codes"):
         saved[name], w = timed(name)
         setattr(ops, name, w)
     torch.cuda.synchronize()
