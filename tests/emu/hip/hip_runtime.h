@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <sched.h>
 #include <thread>
 #include <vector>
 
@@ -42,13 +43,31 @@ template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p 
 // a 3-CU device: the persistent kernels then run few workgroups with several work items each
 inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 3; return hipSuccess; }
 
+// Barrier for heavily oversubscribed threads (256 per workgroup on a few cores): waiters give up the core instead of
+// sleeping on a futex, which costs two system calls and a wake-up per thread and barrier.
+struct EmuBarrier {
+  explicit EmuBarrier(int n_) : n(n_) {}
+  void arrive_and_wait() {
+    const unsigned g = gen.load(std::memory_order_acquire);
+    if (count.fetch_add(1, std::memory_order_acq_rel) + 1 == n) {
+      count.store(0, std::memory_order_relaxed);
+      gen.fetch_add(1, std::memory_order_release);
+    } else {
+      while (gen.load(std::memory_order_acquire) == g) sched_yield();
+    }
+  }
+  const int n;
+  std::atomic<int> count{0};
+  std::atomic<unsigned> gen{0};
+};
+
 struct EmuWave {
-  std::barrier<> bar{64};
+  EmuBarrier bar{64};
   alignas(64) unsigned char slot[64][64];
   const void* ptr[64];
 };
 struct EmuBlock {
-  std::barrier<>* bar;
+  EmuBarrier* bar;
 };
 inline thread_local EmuWave* emu_wave = nullptr;
 inline thread_local EmuBlock* emu_block = nullptr;
@@ -77,7 +96,7 @@ inline void emu_launch(K kernel, dim3 grid, dim3 block, A... args) {
   for (unsigned bz = 0; bz < grid.z; bz++)
   for (unsigned by = 0; by < grid.y; by++)
   for (unsigned bx = 0; bx < grid.x; bx++) {
-    std::barrier<> bar(nthreads);
+    EmuBarrier bar((int)nthreads);
     EmuBlock blk{&bar};
     std::unique_ptr<EmuWave[]> waves(new EmuWave[nthreads / 64]);
     std::vector<std::thread> th;
