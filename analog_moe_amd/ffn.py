@@ -79,23 +79,28 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
     k = sel_idx.shape[-1]
     M = T * k
     gen = cfg.noise_std > 0 and cfg.noise_up is None
-    wu = wd = None
+    wu = wd = ir_up = ir_dn = None
     main = torch.cuda.current_stream()
     if cfg.wmax_up is not None:
         wu, wd = cfg.wmax_up, cfg.wmax_down
+        ir_up, ir_dn = ir_tables(input_range, E, cfg)
     elif cfg.out_bound > 0 or gen:
-        # max |W| per expert only reads the weights: it runs next to the expert sort on a second stream
+        # max |W| per expert and the fp32 input-range tables only read parameters: they run next to the expert
+        # sort on a second stream
         side = _side_stream(x.device)
         side.wait_stream(main)
         with torch.cuda.stream(side):
+            ir_up, ir_dn = ir_tables(input_range, E, cfg)
             wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
             wd = ops.weight_abs_max(values, cfg.noise_per_channel)
-        wu.record_stream(main)
-        wd.record_stream(main)
+        for t in (wu, wd, ir_up, ir_dn):
+            if t is not None:
+                t.record_stream(main)
+    else:
+        ir_up, ir_dn = ir_tables(input_range, E, cfg)
     sel_sorted, perm, in_index, offsets = ops.prepare_sel(sel_idx, E, k)
     if wu is not None and cfg.wmax_up is None:
         main.wait_stream(side)
-    ir_up, ir_dn = ir_tables(input_range, E, cfg)
     common = dict(inp_res=cfg.inp_res, out_bound=cfg.out_bound, out_res=cfg.out_res,
                   noise_std=cfg.noise_std if gen else 0.0, ir_by_expert=ir_up is not None)
     # the up-projection also emits the down-projection's DAC image of its result (each row belongs
