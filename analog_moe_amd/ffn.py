@@ -174,17 +174,20 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
             grad_x = ops.ksum(full, k) if k > 1 else full
     grad_gate.record_stream(main)
     grad_x.record_stream(main)
-    grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
-    grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
-    main.wait_stream(side)
     grad_ir = None
     if ir_up is not None and want_ir_grad:
         ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
-        # the two tables of per-expert sums are written where they belong; only columns neither has need a zero
+        # the two tables of per-expert sums are written where they belong; only columns neither has need a zero.
+        # The fill and the down-projection's sums are issued here, where the second stream keeps the GPU busy,
+        # instead of after the join at the end of the step
         make = torch.empty if ntu == ntd else torch.zeros
         grad_ir = make((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
-        ops.segment_sum(irg_up, offsets, E, out=grad_ir[0, :, :ntu])
         ops.segment_sum(irg_dn, offsets, E, out=grad_ir[1, :, :ntd])
+    grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
+    grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
+    main.wait_stream(side)
+    if grad_ir is not None:
+        ops.segment_sum(irg_up, offsets, E, out=grad_ir[0, :, :ntu])
     return grad_x, grad_keys, grad_values, grad_ir, grad_gate
 
 
