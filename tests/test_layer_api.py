@@ -303,6 +303,28 @@ def test_library_rejects_bad_arguments_on_the_host():
     assert lib.amoe_gate_grad(5, p, p, p, 4, 2, 8, None) == EINVAL
     assert lib.amoe_row_abs_max(_abi.AMOE_F32, p, 4, 8, 16, p, None) == EINVAL          # ldx < K
     assert lib.amoe_weight_abs_max(_abi.AMOE_F32, p, 2, 8, 16, 3, p, None) == EINVAL   # cols is 1 or N
+    # sum over the heads with the input-range clip
+    def ksc(**kw):
+        a = _abi.KsumClipArgs(dtype=_abi.AMOE_F32, T=4, k=2, D=32, E=2, full=p, x=p, ldx=32, sel=p, sel_is_i64=1,
+                              perm=p, offsets=p, ir=p, n_tiles=1, grad_x=p, ir_grad=p, workspace=p,
+                              workspace_bytes=8192)
+        a.tile_bounds[0], a.tile_bounds[1] = 0, 32
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+    assert lib.amoe_ksum_clip(None, None) == ENULL
+    assert lib.amoe_ksum_clip(ksc(dtype=5), None) == EINVAL
+    assert lib.amoe_ksum_clip(ksc(k=0), None) == EINVAL
+    assert lib.amoe_ksum_clip(ksc(T=0), None) == 0                                       # no tokens: nothing to do
+    assert lib.amoe_ksum_clip(ksc(ir=None), None) == ENULL
+    assert lib.amoe_ksum_clip(ksc(ldx=16), None) == ESHAPE
+    assert lib.amoe_ksum_clip(ksc(x=p + 4), None) == EALIGN
+    assert lib.amoe_ksum_clip(ksc(k=9), None) == EUNSUPPORTED                            # more than 8 heads
+    two = ksc(n_tiles=2)
+    two.tile_bounds[1], two.tile_bounds[2] = 18, 32                                      # a bound inside a 16-byte chunk
+    assert lib.amoe_ksum_clip(two, None) == EUNSUPPORTED
+    assert lib.amoe_ksum_clip(ksc(workspace_bytes=16), None) == EWORKSPACE
+    assert lib.amoe_ksum_clip_workspace(4, 2, 1) >= 4 * 2 * 4
     # weight modifier / clip
     F = _abi.AMOE_F32
     assert lib.amoe_modify_weight(F, p, 2, 8, 16, p, 3, 14.0, 0.0, None, 1, 0, None, p, None) == EINVAL    # wmax cols
