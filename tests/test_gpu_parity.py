@@ -127,7 +127,7 @@ def test_wide_kernels_with_uneven_experts(ops, dtype):
     (torch.float32, dict(T=700, D=96, k=3, bounds=[0, 32, 96])),
     (torch.float32, dict(T=2100, D=260, k=2, E=2, strided_x=True, decay=0.0)),
     (torch.bfloat16, dict(T=3000, D=1024, N=64, k=8, E=16, bounds=[0, 512, 1024], sel_dtype=torch.int32)),
-    (torch.bfloat16, dict(T=9000, D=256, N=32, k=4, E=7)),          # more tokens than one round of the grid takes
+    (torch.bfloat16, dict(T=9000, D=256, N=32, k=4, E=7)),          # more tokens than one pass of the grid takes
     (torch.float16, dict(T=1033, D=136, k=4, strided_x=True, input_min_percentage=0.99)),
 ])
 def test_head_sum_with_input_range_clip(ops, dtype, kw):
