@@ -9,6 +9,7 @@ constexpr int kThreads = 256;   // 4 waves per workgroup, arranged 2 x 2 over th
 constexpr int kTileRows = 128;  // token rows per workgroup tile
 constexpr int kTileCols = 128;  // feature columns per workgroup tile
 constexpr int kMaxTiles = 16;
+constexpr int kSelMaxExperts = 2048;   // experts the sort, the per-expert tables and their LDS copies are sized for
 
 // Bit casts through by-value helpers (a bit cast applied directly to a vector element
 // reads element 0 with this compiler).

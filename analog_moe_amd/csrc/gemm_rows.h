@@ -891,15 +891,21 @@ struct IrFinalizeParams {
 
 __global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFinalizeParams p) {
   __shared__ long long sTot[4];
+  __shared__ int sOff[kSelMaxExperts];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  float flag = 0.f;
-  if (p.decay > 0.f) {
-    long long c = 0;
+  // the segment starts come to LDS in the same round trip as the counts: the search below then runs on LDS
+  // instead of on a chain of dependent global loads (E <= kSelMaxExperts: the entry points check it)
+  if (p.ir_by_expert)
+    for (int i = tid; i < p.E; i += kThreads) sOff[i] = p.offsets[i];
+  long long c = 0;
+  if (p.decay > 0.f)
     for (int i = tid; i < p.n_blocks; i += kThreads) c += p.notclip_count[i];
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) c += wave_shfl_xor(c, d);
-    if (lane == 0) sTot[wave] = c;
-    __syncthreads();
+  for (int d = 32; d >= 1; d >>= 1) c += wave_shfl_xor(c, d);
+  if (lane == 0) sTot[wave] = c;
+  __syncthreads();
+  float flag = 0.f;
+  if (p.decay > 0.f) {
     const long long tot = sTot[0] + sTot[1] + sTot[2] + sTot[3];
     const float pct = (float)tot / (float)((long long)p.M * (long long)p.KD_total);
     flag = pct > p.min_pct ? 1.f : 0.f;
@@ -911,7 +917,7 @@ __global__ __launch_bounds__(kThreads) void ir_grad_finalize_kernel(const IrFina
     int lo = 0, hi = p.E - 1;
     while (lo < hi) {
       const int mid = (lo + hi + 1) >> 1;
-      if (p.offsets[mid] <= r) lo = mid; else hi = mid - 1;
+      if (sOff[mid] <= r) lo = mid; else hi = mid - 1;
     }
     ir_row = lo;
   }

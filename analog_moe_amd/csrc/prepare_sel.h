@@ -18,7 +18,6 @@ __host__ __device__ inline int sel_unit(long long M) {
   while (u < kSelUnitMax && M / u > 2048) u <<= 1;   // aim at <= 2048 units
   return u < 256 ? 256 : u;
 }
-constexpr int kSelMaxExperts = 2048;
 
 struct SelParams {
   const void* sel; int sel_is_i64;
