@@ -62,6 +62,7 @@ def test_counter_runs_become_bytes_per_launch(tmp_path, monkeypatch):
 def test_recorded_traffic_file_is_well_formed():
     path = BT.traffic_file("c3")
     assert os.path.exists(path)
-    rec = json.load(open(path))
+    with open(path) as fh:
+        rec = json.load(fh)
     assert set(rec["launches"]) == {"fwd_up", "fwd_down", "xgrad_down", "xgrad_up", "wgrad_down", "wgrad_up"}
     assert all(v["total_bytes"] > 1e8 for v in rec["launches"].values())

@@ -677,7 +677,7 @@ def test_regulariser_and_select_bwd_match_torch_autograd():
     gv = torch.randn(50, 3)
     ((val * gv).sum() + 0.7 * reg).backward()
     got_reg, c = SO.usage_regulariser(logits.detach().numpy())
-    assert abs(float(got_reg) - float(reg)) < 1e-6
+    assert abs(float(got_reg) - float(reg.detach())) < 1e-6
     uniform_reg, _ = SO.usage_regulariser(np.zeros((7, 8), np.float32))
     assert abs(float(uniform_reg) + np.log(8)) < 1e-6                       # uniform usage: minus log E
     got = SO.select_bwd(logits.detach().numpy(), idx.numpy(), gv.numpy(), 0.7)
