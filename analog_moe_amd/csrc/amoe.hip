@@ -815,6 +815,39 @@ static ColSplit col_split(int dtype, int E, int K, int N) {
   return c;
 }
 
+int amoe_weight_abs_max_pair(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a,
+                             const void* w_b, int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, void* stream) {
+  if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
+  if (E < 1 || K_a < 1 || N_a < 1 || K_b < 1 || N_b < 1) return AMOE_EINVAL;
+  if (!w_a || !w_b || !wmax_a || !wmax_b) return AMOE_ENULL;
+  if (!aligned(w_a, esize(dtype)) || !aligned(w_b, esize(dtype)) || !aligned(wmax_a, 4) || !aligned(wmax_b, 4))
+    return AMOE_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const long long per_a = (long long)K_a * N_a, per_b = (long long)K_b * N_b;
+  const long long per = per_a > per_b ? per_a : per_b;
+  int chunks = (int)((per + 32 * kThreads - 1) / (32 * kThreads));
+  chunks = chunks < 1 ? 1 : (chunks > 64 ? 64 : chunks);
+  const int vec_a = aligned(w_a, 16) && (per_a % 16 == 0), vec_b = aligned(w_b, 16) && (per_b % 16 == 0);
+  hipLaunchKernelGGL(fill_zero2_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
+                     reinterpret_cast<uint32_t*>(wmax_a), (int)E, reinterpret_cast<uint32_t*>(wmax_b), (int)E);
+  if (int rc = launch_rc()) return rc;
+  const dim3 grid(chunks, E, 2);
+  if (dtype == AMOE_F32) {
+    auto kf = &weight_abs_max_kernel<float>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const float*>(w_a), per_a, wmax_a, vec_a,
+                       static_cast<const float*>(w_b), per_b, wmax_b, vec_b);
+  } else if (dtype == AMOE_BF16) {
+    auto kf = &weight_abs_max_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(w_a), per_a, wmax_a, vec_a,
+                       static_cast<const uint16_t*>(w_b), per_b, wmax_b, vec_b);
+  } else {
+    auto kf = &weight_abs_max_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, static_cast<const f16_t*>(w_a), per_a, wmax_a, vec_a,
+                       static_cast<const f16_t*>(w_b), per_b, wmax_b, vec_b);
+  }
+  return launch_rc();
+}
+
 int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N, int32_t cols, float* wmax,
                         void* stream) {
   if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
@@ -832,13 +865,16 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
     if (int rc = launch_rc()) return rc;
     if (dtype == AMOE_F32) {
       auto kf = &weight_abs_max_kernel<float>;
-      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax, vec);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const float*>(w), per, wmax, vec,
+                         static_cast<const float*>(nullptr), 0LL, static_cast<float*>(nullptr), 0);
     } else if (dtype == AMOE_BF16) {
       auto kf = &weight_abs_max_kernel<uint16_t>;
-      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax, vec);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const uint16_t*>(w), per, wmax, vec,
+                         static_cast<const uint16_t*>(nullptr), 0LL, static_cast<float*>(nullptr), 0);
     } else {
       auto kf = &weight_abs_max_kernel<f16_t>;
-      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const f16_t*>(w), per, wmax, vec);
+      hipLaunchKernelGGL(kf, dim3(chunks, E), dim3(kThreads), 0, st, static_cast<const f16_t*>(w), per, wmax, vec,
+                         static_cast<const f16_t*>(nullptr), 0LL, static_cast<float*>(nullptr), 0);
     }
   } else if (dtype == AMOE_BF16) {
     if ((long long)E * N > 0x7fffffffLL) return AMOE_EUNSUPPORTED;

@@ -370,11 +370,22 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restric
   const int i = blockIdx.x * kThreads + threadIdx.x;
   if (i < n) p[i] = 0u;
 }
+__global__ __launch_bounds__(kThreads) void fill_zero2_kernel(uint32_t* __restrict__ a, int na,
+                                                               uint32_t* __restrict__ b, int nb) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < na) a[i] = 0u;
+  if (i < nb) b[i] = 0u;
+}
+// (blockIdx.z picks one of two weight tensors of the same expert count: both tables of a layer from one launch)
 template <typename T>
 __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __restrict__ w, long long per_expert,
-                                                                   float* __restrict__ out, int vec) {
+                                                                   float* __restrict__ out, int vec,
+                                                                   const T* __restrict__ w2 = nullptr,
+                                                                   long long per_expert2 = 0,
+                                                                   float* __restrict__ out2 = nullptr, int vec2 = 0) {
   __shared__ float red[4];
   const int tid = threadIdx.x, lane = tid & 63;
+  if (blockIdx.z == 1) { w = w2; per_expert = per_expert2; out = out2; vec = vec2; }
   const T* base = w + (long long)blockIdx.y * per_expert;
   long long span = (per_expert + gridDim.x - 1) / gridDim.x;
   span = (span + 15) / 16 * 16;             // keep slices 16-byte aligned

@@ -91,8 +91,11 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
         side.wait_stream(main)
         with torch.cuda.stream(side):
             ir_up, ir_dn = ir_tables(input_range, E, cfg)
-            wu = ops.weight_abs_max(keys, cfg.noise_per_channel)
-            wd = ops.weight_abs_max(values, cfg.noise_per_channel)
+            if cfg.noise_per_channel:
+                wu = ops.weight_abs_max(keys, True)
+                wd = ops.weight_abs_max(values, True)
+            else:
+                wu, wd = ops.weight_abs_max_pair(keys, values)
         for t in (wu, wd, ir_up, ir_dn):
             if t is not None:
                 t.record_stream(main)

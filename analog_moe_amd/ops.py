@@ -302,6 +302,16 @@ def weight_abs_max(w: torch.Tensor, per_channel: bool) -> torch.Tensor:
     return out
 
 
+def weight_abs_max_pair(w_a: torch.Tensor, w_b: torch.Tensor):
+    """Per-expert max |w| of two weight tensors of one layer ([E, 1] fp32 each) from one pair of launches."""
+    _need_gpu(w_a, w_b)
+    a, b = w_a.detach().contiguous(), w_b.detach().contiguous()
+    E = a.shape[0]
+    both = torch.empty((2, E, 1), dtype=torch.float32, device=a.device)
+    raw.weight_abs_max_pair(get_lib(), _stream(a), a, b, both[0], both[1])
+    return both[0], both[1]
+
+
 def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[e, t] = sum of v[i, t] over expert e's sorted rows.  ``out``: fp32 [E, columns of v] to write into (its

@@ -274,6 +274,15 @@ def weight_abs_max(lib, stream, w, cols: int, out):
           "amoe_weight_abs_max")
 
 
+def weight_abs_max_pair(lib, stream, w_a, w_b, out_a, out_b):
+    if not w_a.is_contiguous() or not w_b.is_contiguous() or w_a.dtype != w_b.dtype or w_a.shape[0] != w_b.shape[0]:
+        raise ValueError("two contiguous weight tensors of one dtype and one expert count")
+    E = w_a.shape[0]
+    check(lib, lib.amoe_weight_abs_max_pair(dtype_code(w_a), _p(w_a), w_a.shape[1], w_a.shape[2],
+                                            _p(_f32(out_a, "wmax_a")), _p(w_b), w_b.shape[1], w_b.shape[2],
+                                            _p(_f32(out_b, "wmax_b")), E, stream), "amoe_weight_abs_max_pair")
+
+
 def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out):
     """out: fp32 [E, n_tiles], rows any stride apart (a slice of a wider table will do)"""
     if (out.dtype != torch.float32 or out.dim() != 2 or tuple(out.shape) != (E, n_tiles) or

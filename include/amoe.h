@@ -287,6 +287,11 @@ int amoe_row_abs_max(int32_t dtype, const void* x, int64_t ldx, int64_t rows, in
  * (moe_layer_aihwkit_lightning.py:480-487) */
 int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int32_t N,
                         int32_t cols, float* wmax, void* stream);
+/* Both per-expert tables of a layer, wmax_a[e] = max |w_a[e]| and wmax_b[e] = max |w_b[e]| (the cols == 1 case of
+ * amoe_weight_abs_max for keys [E, K_a, N_a] and values [E, K_b, N_b]), from one zero fill and one reduction
+ * launch instead of two of each (moe_layer_aihwkit_lightning.py:480-487, once per projection there). */
+int amoe_weight_abs_max_pair(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a,
+                             const void* w_b, int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, void* stream);
 /* out[e * ldout + t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]
  * (moe_layer_aihwkit_lightning.py:447-448), fixed order.  ldout >= n_tiles: the row stride of out, so that the
  * sums can land in a slice of a wider table. */

@@ -176,6 +176,9 @@ def test_companions(emu_ops):
     assert torch.equal(emu_ops.weight_abs_max(pr["keys"], False), pr["keys"].abs().amax((1, 2)).reshape(5, 1))
     assert torch.equal(emu_ops.weight_abs_max(pr["keys"], True), pr["keys"].abs().amax(1))
     util.check_weight_abs_max(emu_ops)
+    va = pr["values"].to(torch.float16)[:, :, :61].contiguous()                      # 20 x 61: no 16-byte slices
+    wa, wb = emu_ops.weight_abs_max_pair(pr["keys"].to(torch.float16), va)
+    assert torch.equal(wb, va.float().abs().amax((1, 2)).reshape(5, 1))
     s = emu_ops.prepare_sel(pr["idx"].clamp(max=3), 5, 2)
     std = emu_ops.expert_std(x, s[2], s[3], 5)
     want = O.expert_std(x.numpy(), s[2].numpy(), s[0].numpy(), 5)

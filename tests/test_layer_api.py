@@ -303,6 +303,9 @@ def test_library_rejects_bad_arguments_on_the_host():
     assert lib.amoe_gate_grad(5, p, p, p, 4, 2, 8, None) == EINVAL
     assert lib.amoe_row_abs_max(_abi.AMOE_F32, p, 4, 8, 16, p, None) == EINVAL          # ldx < K
     assert lib.amoe_weight_abs_max(_abi.AMOE_F32, p, 2, 8, 16, 3, p, None) == EINVAL   # cols is 1 or N
+    assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p, p, 0, 8, p, 2, None) == EINVAL
+    assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p, None, 16, 8, p, 2, None) == ENULL
+    assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p + 2, p, 16, 8, p, 2, None) == EALIGN
     # sum over the heads with the input-range clip
     def ksc(**kw):
         a = _abi.KsumClipArgs(dtype=_abi.AMOE_F32, T=4, k=2, D=32, E=2, full=p, x=p, ldx=32, sel=p, sel_is_i64=1,

@@ -500,6 +500,11 @@ def check_weight_abs_max(ops, device="cpu"):
         w = modifier_weights(E + K, E, K, N, dtype, device)
         assert torch.equal(ops.weight_abs_max(w, True), w.abs().amax(1).float()), (E, K, N)
         assert torch.equal(ops.weight_abs_max(w, False), w.abs().amax((1, 2)).float().reshape(E, 1)), (E, K, N)
+        # both tables of a layer from one pair of launches: this tensor and its transposed twin of other values
+        w2 = (modifier_weights(E + K + 1, E, N, K, dtype, device) * 3).to(dtype)
+        wa, wb = ops.weight_abs_max_pair(w, w2)
+        assert torch.equal(wa, w.abs().amax((1, 2)).float().reshape(E, 1)), (E, K, N)
+        assert torch.equal(wb, w2.abs().amax((1, 2)).float().reshape(E, 1)), (E, K, N)
 
 
 # ---------------------------------------------------------------------------------- router epilogue
