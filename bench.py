@@ -321,7 +321,8 @@ def main():
         spin_cycles = int(2.0 / max(s0.elapsed_time(e0), 1e-3) * 1_000_000)
     saved = {}
     for name in ("cvmm_fwd", "cvmm_bwd_w", "cvmm_bwd_x", "prepare_sel", "gate_reduce", "gate_grad", "ksum",
-                 "ksum_clip", "weight_abs_max", "segment_sum", "gate_reduce_codes", "gate_grad_codes"):
+                 "ksum_clip", "weight_abs_max", "weight_abs_max_pair", "segment_sum", "gate_reduce_codes",
+                 "gate_grad_codes"):
         saved[name], w = timed(name)
         setattr(ops, name, w)
     torch.cuda.synchronize()
