@@ -84,6 +84,7 @@ PROTOTYPES = {
     "amoe_prepare_sel_noalloc": (C.c_int, [P, I32, I64, I32, I32, P, P, P, P, P, P]),
     "amoe_offsets_from_sorted": (C.c_int, [P, I64, I32, P, P]),
     "amoe_cvmm_fwd": (C.c_int, [C.POINTER(FwdArgs), P]),
+    "amoe_fwd_codes_supported": (C.c_int, [C.POINTER(FwdArgs)]),
     "amoe_bwd_w_workspace": (SZ, [C.POINTER(BwdWArgs)]),
     "amoe_cvmm_bwd_w": (C.c_int, [C.POINTER(BwdWArgs), P]),
     "amoe_bwd_x_workspace": (SZ, [I64, I32, I32]),

@@ -35,6 +35,11 @@ inline bool bounds_multiple_of(int n_tiles, const int32_t* b, int m) {
   return true;
 }
 inline size_t esize(int dtype) { return dtype == AMOE_F32 ? 4 : 2; }
+// Whether every DAC code of a quantiser with step inp_res (codes -1/inp_res .. 1/inp_res) is exact in the type.
+inline bool dac_codes_fit(int dtype, float inp_res) {
+  if (dtype == AMOE_F32 || !(inp_res > 0.f)) return true;
+  return 1.0f / inp_res <= (dtype == AMOE_BF16 ? 256.f : 2048.f) * (1.0f + 1e-6f);
+}
 inline int max_row_tiles(int64_t M, int E) { return (int)(M / kTileRows) + E; }
 
 // Compute units of the current device (read once; the value cannot change while the process lives).
@@ -108,6 +113,13 @@ int launch_fwd256_as(const RowsParams& p, int grid, hipStream_t st) {
   return launch_rc();
 }
 
+// The input gradient reads the forward input x (through xf_index) only for the features that need it: the
+// input-range clip, the ReLU mask, the clipped-input output.  A caller that passes x without any of them has not
+// been asked for xf_index, and its launch is a plain product.
+inline bool bwdx_reads_x(const amoe_bwd_x_args* a) {
+  return a->x != nullptr && a->xf_index != nullptr && (a->ir != nullptr || a->relu_mask != 0 || a->xc_out != nullptr);
+}
+
 // The 128 x 256 input-gradient kernel, for the same launches (and column tiles that are multiples of 256).  The
 // partial sums of the input-range gradient then cover 256 columns each; *n_count_blocks is the grid that ran.
 template <typename T, int COLS>
@@ -116,7 +128,7 @@ int launch_bwdx256_cols(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, 
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks, COLS == 128 ? 3 : 2);
   *n_count_blocks = grid;
   const bool relu = a->relu_mask != 0, xc = a->xc_out != nullptr;
-  if (a->x == nullptr) {
+  if (!bwdx_reads_x(a)) {
     hipLaunchKernelGGL((&bwdx256_kernel<T, false, false, false, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
   } else if (!relu) {
     if (xc) hipLaunchKernelGGL((&bwdx256_kernel<T, true, false, true, COLS>), dim3(grid), dim3(kThreads), 0, st, p);
@@ -135,7 +147,7 @@ int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* 
   if (a->x != nullptr && (!aligned(a->x, 16) || a->ldx % 8)) return AMOE_EUNSUPPORTED;   // 16-byte pieces of x rows
   // With a short contraction an item is mostly its mask stage: 128-column tiles at three workgroups per CU then
   // hide more of it (C3's up-projection, contraction 256: 0.197 vs 0.212 ms; at 512 the wide tile wins again).
-  const bool narrow = a->x != nullptr && a->N <= 256;
+  const bool narrow = bwdx_reads_x(a) && a->N <= 256;
   const int cols = narrow ? 128 : kFCols;
   for (int t = 0; t < a->n_tiles; t++)
     if ((a->tile_bounds[t + 1] - a->tile_bounds[t]) % cols) return AMOE_EUNSUPPORTED;
@@ -154,6 +166,9 @@ int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st
   const bool analog = adc && a->out_res > 0.f && a->wmax_cols == 1 && dac;
   if ((adc || noisy) && !analog) return AMOE_EUNSUPPORTED;
   if (a->n_tiles == 2 && !(analog && !a->x_is_quantized)) return AMOE_EUNSUPPORTED;
+  // the two-K-tile variant parks the first tile's ADC codes as bytes (code + 128): a finer output quantiser than
+  // 254 states does not fit them, and the general kernel (fp32 partial results) serves the launch
+  if (a->n_tiles == 2 && !(p.out_half_states <= 127.f)) return AMOE_EUNSUPPORTED;
   p.n_col_blocks = a->N / kFCols;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
   if (a->code_out && !analog) return AMOE_EUNSUPPORTED;
@@ -163,9 +178,7 @@ int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st
                              : launch_fwd256_as<T, FA_DAC, false, false, false>(p, grid, st);
   if (a->code_out) {
     // codes leave instead of values: one output quantiser whose half range fits a byte, no second output
-    const float half = 0.5f * fmaxf(a->out_res, 1.0f / a->out_res);
-    if (a->n_tiles != 1 || a->xq_out || a->relu || !(half <= 127.f) || !aligned(a->code_out, 16) || a->ldcode % 16)
-      return AMOE_EUNSUPPORTED;
+    if (!amoe_fwd_codes_supported(a) || !aligned(a->code_out, 16)) return AMOE_EUNSUPPORTED;
     if (a->x_is_quantized)
       return noisy ? launch_fwd256_as<T, FA_CODES, true, true, false, true>(p, grid, st)
                    : launch_fwd256_as<T, FA_CODES, true, false, false, true>(p, grid, st);
@@ -302,6 +315,25 @@ int amoe_offsets_from_sorted(const int32_t* sel_sorted, int64_t M, int32_t E, in
 }
 
 // ------------------------------------------------------------------------------ forward
+int amoe_fwd_codes_supported(const amoe_fwd_args* a) {
+  if (!a || (a->dtype != AMOE_BF16 && a->dtype != AMOE_F16)) return 0;
+  if (a->N < 1 || a->K < 1 || a->E < 1 || a->n_tiles != 1 || a->w_stride_n != 1) return 0;
+  // every tile interior, 16-byte pieces everywhere, 32-bit byte offsets
+  if (a->N % kFCols || a->K % kFBK || a->ldx % 8 || a->w_stride_e % 8 || a->w_stride_k % 8 || a->ldcode % 16) return 0;
+  if (a->ldx < a->K || a->w_stride_k < a->N || a->ldcode < a->N) return 0;
+  const long long lim = 1LL << 31;
+  if (a->n_in_rows <= 0 || (long long)a->n_in_rows * a->ldx * 2 >= lim ||
+      ((long long)a->K * a->w_stride_k + (long long)a->N) * 2 >= lim)
+    return 0;
+  // the analog stages the kernel is built for: per-expert input ranges with an input quantiser whose codes the type
+  // holds, one max |W| per expert, generated noise or none, an output quantiser whose codes fit a byte
+  if (!a->ir || !a->ir_by_expert || !(a->inp_res > 0.f) || !dac_codes_fit(a->dtype, a->inp_res) || a->abs_max) return 0;
+  if (a->noise || !a->wmax || a->wmax_cols != 1 || !(a->out_bound > 0.f) || !(a->out_res > 0.f)) return 0;
+  if (!(0.5f * fmaxf(a->out_res, 1.0f / a->out_res) <= 127.f)) return 0;
+  if (a->xq_out || a->relu) return 0;
+  return 1;
+}
+
 int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   if (!a) return AMOE_ENULL;
   if (a->dtype != AMOE_F32 && a->dtype != AMOE_BF16 && a->dtype != AMOE_F16) return AMOE_EINVAL;
@@ -319,6 +351,10 @@ int amoe_cvmm_fwd(const amoe_fwd_args* a, void* stream) {
   if (a->xq_out && (!a->xq_ir || !(a->xq_inp_res > 0.f))) return AMOE_EINVAL;
   if (a->xq_out && a->ldxq < a->N) return AMOE_ESHAPE;
   if (a->x_is_quantized && (!a->ir || !(a->inp_res > 0.f) || a->abs_max || a->n_tiles != 1)) return AMOE_EINVAL;
+  // 16-bit element types carry the DAC codes themselves to the matrix unit (and in xq_out): integers are exact up
+  // to 256 in bf16 and 2048 in fp16, so a finer input quantiser needs fp32 tensors
+  if (!dac_codes_fit(a->dtype, a->inp_res) || (a->xq_out && !dac_codes_fit(a->dtype, a->xq_inp_res)))
+    return AMOE_EUNSUPPORTED;
   const size_t es = esize(a->dtype);
   if (!aligned(a->x, es) || !aligned(a->w, es) || !aligned(a->out, es) || !aligned(a->offsets, 4) ||
       !aligned(a->in_index, 4) || !aligned(a->out_index, 4) || !aligned(a->ir, 4) || !aligned(a->abs_max, 4) ||

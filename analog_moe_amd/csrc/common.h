@@ -185,7 +185,8 @@ __device__ __forceinline__ Raw raw_pack_exact_bf16(const float (&v)[8]) {
   for (int j = 0; j < 4; j++) r[j] = (as_u32(v[2 * j]) >> 16) | (as_u32(v[2 * j + 1]) & 0xffff0000u);
   return r;
 }
-// small integers (DAC codes) as 16-bit elements of T: exact in bf16 and in fp16
+// DAC codes as 16-bit elements of T.  Exact only while the type holds the integers: |code| <= 256 in bf16 (the
+// truncation below drops nothing then), <= 2048 in fp16; the host rejects finer input quantisers for these types.
 template <typename T>
 __device__ __forceinline__ Raw raw_pack_codes(const float (&v)[8]) {
   if constexpr (kIsF16<T>) return raw_pack<T>(v);

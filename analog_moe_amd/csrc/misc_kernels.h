@@ -144,8 +144,10 @@ __global__ __launch_bounds__(kThreads) void head_reduce_codes_kernel(const uint8
 }
 
 // grad_gate[t*k+j] = <z[t*k+j, :], dy[t, :]>.  A wave takes kCodeTokens tokens at once (their loads are all in
-// flight together); a lane owns runs of 16 columns.  sum (c - 128) * dy = sum c * dy - 128 * sum dy: the products
-// run on the bytes as they are, the row's two scale factors multiply the finished sum.  D % 16 == 0.
+// flight together); a lane owns runs of 16 columns.  Each term (c - 128) * dy is formed as fma(c, dy, -128 * dy) on
+// the byte as it is: -128 * dy is exact, so the fused operation rounds the exact product (c - 128) * dy once, as a
+// multiplication by the signed code would (no large common part that cancels afterwards).  The row's two scale
+// factors multiply the finished sum.  D % 16 == 0.
 constexpr int kCodeTokens = 2;
 template <typename T>
 __global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t* __restrict__ codes,
@@ -158,10 +160,9 @@ __global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t
   const long long t0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * TK;
   if (t0 >= tokens) return;
   for (int j0 = 0; j0 < k; j0 += JB) {
-    float s[TK][JB], sb[TK];
+    float s[TK][JB];
 #pragma unroll
     for (int u = 0; u < TK; u++) {
-      sb[u] = 0.f;
 #pragma unroll
       for (int jj = 0; jj < JB; jj++) s[u][jj] = 0.f;
     }
@@ -193,26 +194,23 @@ __global__ __launch_bounds__(kThreads) void gate_grad_codes_kernel(const uint8_t
 #pragma unroll
             for (int i = 0; i < 4; i++) b[4 * q + i] = as_f32(rd[u][q][i]);
         }
-        float bs = 0.f;
+        float nb[16];
 #pragma unroll
-        for (int q = 0; q < 16; q++) bs += b[q];
-        sb[u] += bs;
+        for (int q = 0; q < 16; q++) nb[q] = -128.0f * b[q];
 #pragma unroll
         for (int jj = 0; jj < JB; jj++) {
           float acc = 0.f;
 #pragma unroll
           for (int w = 0; w < 4; w++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc += (float)((rc[u][jj][w] >> (8 * i)) & 0xffu) * b[4 * w + i];
+            for (int i = 0; i < 4; i++)
+              acc += fmaf((float)((rc[u][jj][w] >> (8 * i)) & 0xffu), b[4 * w + i], nb[4 * w + i]);
           s[u][jj] += acc;
         }
       }
     }
 #pragma unroll
     for (int u = 0; u < TK; u++) {
-      // the offset leaves before the lanes meet (128 * sum dy is exact in every lane), then eight sums in one pass
-#pragma unroll
-      for (int jj = 0; jj < JB; jj++) s[u][jj] -= 128.0f * sb[u];
       const float v = wave_sum8(s[u], lane);
       const int jj = lane >> 3;
       if ((lane & 7) == 0 && j0 + jj < k && t0 + u < tokens) {

@@ -129,18 +129,31 @@ def cvmm_fwd(x: torch.Tensor, w: torch.Tensor, sel_sorted: torch.Tensor, offsets
 
 def codes_supported(x: torch.Tensor, w: torch.Tensor, *, ir_by_expert: bool, inp_res: float, n_tiles: int,
                     out_bound: float, out_res: float, noise: Optional[torch.Tensor], per_channel: bool) -> bool:
-    """Whether ``cvmm_fwd(..., want_codes=True)`` has a kernel for this call: the 128 x 256 forward kernel
-    with an output quantiser of at most 254 states (bf16 or fp16, every tile interior: N a multiple of 256, K of 32,
-    16-byte aligned rows; per-expert input ranges with input quantisation; one max |W| per expert; no injected
-    noise; one K-tile).  A pure function of shapes and settings, so that traced code can rely on it."""
-    if x.dtype not in (torch.bfloat16, torch.float16) or w.dtype != x.dtype or not w.is_contiguous():
+    """Whether ``cvmm_fwd(..., want_codes=True)`` has a kernel for this call.  The library decides
+    (``amoe_fwd_codes_supported``, the same function its launcher asks); only shapes, strides and settings are
+    passed, so the answer is a pure function of them and holds for meta tensors under a tracer too.  x and w as
+    ``cvmm_fwd`` would hand them over (freshly allocated tensors are 16-byte aligned, which is all that is left)."""
+    if x.dtype not in (torch.bfloat16, torch.float16) or w.dtype != x.dtype or w.dim() != 3:
         return False
     E, K, N = w.shape
-    x2_stride = x.stride(-2) if x.dim() >= 2 else K
-    half = 0.5 * max(out_res, 1.0 / out_res) if out_res > 0 else 0.0
-    return (ir_by_expert and inp_res > 0 and n_tiles == 1 and out_bound > 0 and 0 < half <= 127 and noise is None
-            and not per_channel and N % 256 == 0 and K % 32 == 0 and x2_stride % 8 == 0 and x.stride(-1) == 1
-            and x.numel() * 2 < 2 ** 31 and (K * N) * 2 < 2 ** 31)
+    if x.dim() < 2 or x.shape[-1] != K or x.stride(-1) != 1 or (w.stride(2) != 1 and w.stride(1) != 1):
+        return False
+    a = _abi.FwdArgs()
+    a.dtype = raw.dtype_code(x)
+    a.M, a.N, a.K, a.E = 1, N, K, E
+    a.n_in_rows = x.numel() // K
+    a.ldx = x.stride(-2)
+    a.w_stride_e, a.w_stride_k, a.w_stride_n = w.stride(0), w.stride(1), w.stride(2)
+    _abi.set_bounds(a, [0, K])
+    a.n_tiles = n_tiles
+    flag = 1                       # pointer fields are read as present / absent only
+    a.ir, a.ir_by_expert = (flag if ir_by_expert else None), int(bool(ir_by_expert))
+    a.inp_res = float(inp_res)
+    a.noise = flag if noise is not None else None
+    a.wmax, a.wmax_cols = flag, (N if per_channel else 1)
+    a.out_bound, a.out_res = float(out_bound), float(out_res)
+    a.code_out, a.ldcode, a.code_scale_out = flag, N, flag
+    return bool(get_lib().amoe_fwd_codes_supported(a))
 
 
 def cvmm_bwd_w(x: torch.Tensor, g: torch.Tensor, n_experts: int, offsets: torch.Tensor, in_index: torch.Tensor,

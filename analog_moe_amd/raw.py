@@ -122,6 +122,14 @@ def cvmm_fwd(lib, stream, x, w, out, sel_sorted, offsets, in_index, out_index=No
             raise ValueError("xq_out must match out")
         a.xq_out, a.ldxq, a.xq_ir, a.xq_inp_res = _p(xq_out), xq_out.stride(0), _p(_f32(xq_ir, "xq_ir")), float(xq_inp_res)
     a.x_is_quantized = int(bool(x_is_quantized))
+    if x.dtype != torch.float32:
+        # the 16-bit kernels feed the DAC codes themselves to the matrix unit: integers are exact up to 256 in
+        # bf16 and 2048 in fp16 (the library returns AMOE_EUNSUPPORTED beyond that; say why here)
+        most = 256 if x.dtype == torch.bfloat16 else 2048
+        for name, res in (("inp_res", inp_res), ("xq_inp_res", xq_inp_res if xq_out is not None else -1.0)):
+            if res > 0 and 1.0 / res > most * (1 + 1e-6):
+                raise ValueError(f"{name}={res}: an input quantiser with more than {2 * most} steps needs fp32 tensors "
+                                 f"({x.dtype} holds the codes exactly only up to +-{most})")
     check(lib, lib.amoe_cvmm_fwd(C.byref(a), stream), "amoe_cvmm_fwd")
 
 

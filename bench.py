@@ -224,7 +224,7 @@ def main():
     import torch
     from analog_moe_amd import config as cfgmod, ops
     from analog_moe_amd.moe_layer import AnalogSigmaMoELayer
-    from tests import util
+    from analog_moe_amd.synthetic import make_problem
 
     cfg = CONFIGS[args.config]
     if "layers" in cfg:
@@ -250,7 +250,7 @@ def main():
     torch.manual_seed(0)
     layer = AnalogSigmaMoELayer(rpu, d_model=D, n_experts=E, expert_size=F, k=k).to(dev).to(tdt)
     layer.train()
-    pr = util.make_problem(0, T, D, E, F, k, dtype=tdt, routing=cfg["routing"])
+    pr = make_problem(0, T, D, E, F, k, dtype=tdt, routing=cfg["routing"])
     with torch.no_grad():
         layer.keys.copy_(pr["keys"])
         layer.values.copy_(pr["values"])

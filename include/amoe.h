@@ -144,6 +144,15 @@ typedef struct amoe_fwd_args {
 
 int amoe_cvmm_fwd(const amoe_fwd_args* args, void* stream);
 
+/* Whether amoe_cvmm_fwd has a kernel that leaves the result as ADC codes (args->code_out) for a call of these
+ * shapes, strides and settings: 1 or 0.  The one place where that is decided: amoe_cvmm_fwd asks this function
+ * itself, and callers that must know the result's type before the call (operator shape functions under a tracer;
+ * the reference's counterpart is the abstract implementation at cvmm.py:634-642) ask it instead of restating its
+ * rules.  Only sizes, strides and scalars are read; pointer fields count as flags (NULL = feature off) and are
+ * never dereferenced, so placeholders will do.  What remains for the call itself is the 16-byte alignment of x, w
+ * and code_out. */
+int amoe_fwd_codes_supported(const amoe_fwd_args* args);
+
 /* ---------------------------------------------------------------------------------------
  * Weight gradient: grad_w[e] = sum_{i in expert e} clamp(x[in_index[i]], +-ir[i,t])^T
  *                                                   g[g_index[i]]          -> [E, K, N]

@@ -100,6 +100,21 @@ CASES = {
     "f16_wide_split": (dict(T=90, D=512, E=3, F=256, k=2),
                        dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0, out_res=254.0,
                             decay=0.01), "f16", 2e-3),
+    # an output quantiser finer than 8 bits (1022 states): its codes do not fit the bytes in which the two-K-tile
+    # variant of the 128 x 256 forward kernel parks the first tile, nor the byte-coded result; those launches must
+    # fall to the kernels that keep fp32 values.  Per-expert ranges, so that the wide kernels are candidates.
+    "bf16_wide_fine_adc_split": (dict(T=90, D=512, E=3, F=256, k=2),
+                                 dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0,
+                                      out_res=1022.0, by_expert=True), "bf16", 2e-2),
+    "bf16_wide_fine_adc": (dict(T=90, D=256, E=3, F=256, k=2),
+                           dict(ir=True, inp_res=1 / 127, out_bound=12.0, out_res=1022.0, by_expert=True), "bf16", 2e-2),
+    "f16_wide_fine_adc_split": (dict(T=90, D=512, E=3, F=256, k=2),
+                                dict(ir=True, inp_res=1 / 127, bounds_up=[0, 256, 512], out_bound=12.0,
+                                     out_res=1.0 / 1022.0, by_expert=True), "f16", 2e-3),
+    # an input quantiser finer than 8 bits (10 bit: codes up to 511) in fp32, and in fp16, which holds them exactly
+    "f32_fine_dac": (dict(T=48, D=128, E=4, F=64, k=2), dict(ir=True, inp_res=2.0 / (2 ** 10 - 2)), "f32", 1e-5),
+    "f16_wide_fine_dac": (dict(T=90, D=256, E=3, F=256, k=2),
+                          dict(ir=True, inp_res=2.0 / (2 ** 10 - 2), by_expert=True), "f16", 2e-3),
 }
 
 
@@ -109,7 +124,7 @@ def test_layer_parity_emulated(emu_ops, name):
     lk = dict(lk)
     # alternate between the per-position input-range vector of the reference and the fused
     # per-expert table / in-kernel gate (x) dy product
-    lk["by_expert"] = list(CASES).index(name) % 2 == 1
+    lk.setdefault("by_expert", list(CASES).index(name) % 2 == 1)
     tdt = util.TORCH_DTYPE[dtype]
     pr = util.make_problem(7, dtype=tdt, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
@@ -243,6 +258,46 @@ def test_transposed_weight_view(emu_ops):
     a16 = emu_ops.cvmm_fwd(pr["x"].bfloat16(), wt16, s_sorted, offsets, in_index, perm, 60)
     b16 = emu_ops.cvmm_fwd(pr["x"].bfloat16(), pr["keys"].bfloat16(), s_sorted, offsets, in_index, perm, 60)
     assert torch.equal(a16, b16)
+
+
+def test_input_quantiser_finer_than_the_element_type_is_rejected(emu_ops):
+    """bf16 holds integers exactly up to 256, fp16 up to 2048: the 16-bit kernels carry the DAC codes themselves, so a
+    finer quantiser must be refused (on the host, before anything is launched) instead of truncating codes."""
+    pr = util.make_problem(1, T=8, D=16, E=2, F=8, k=2, dtype=torch.bfloat16)
+    s_sorted, perm, in_index, offsets = emu_ops.prepare_sel(pr["idx"], 2, 2)
+    ir = torch.ones(2, 1)
+    args = (pr["x"], pr["keys"], s_sorted, offsets, in_index, perm, 16)
+    with pytest.raises(ValueError, match="needs fp32"):
+        emu_ops.cvmm_fwd(*args, ir=ir, ir_by_expert=True, inp_res=2.0 / (2 ** 10 - 2))
+    emu_ops.cvmm_fwd(*args, ir=ir, ir_by_expert=True, inp_res=1.0 / 256)          # the finest bf16 carries
+    with pytest.raises(ValueError, match="xq_inp_res"):
+        emu_ops.cvmm_fwd(*args, ir=ir, ir_by_expert=True, inp_res=1.0 / 127, xq_ir=torch.ones(2), xq_inp_res=1.0 / 511)
+    h = {n: (t.half() if t.is_floating_point() else t) for n, t in pr.items()}
+    argh = (h["x"], h["keys"], s_sorted, offsets, in_index, perm, 16)
+    emu_ops.cvmm_fwd(*argh, ir=ir, ir_by_expert=True, inp_res=1.0 / 2047)
+    with pytest.raises(ValueError, match="needs fp32"):
+        emu_ops.cvmm_fwd(*argh, ir=ir, ir_by_expert=True, inp_res=1.0 / 8191)
+    # and by the library itself, for callers that bypass the Python layer
+    a = _abi.FwdArgs()
+    a.dtype, a.M, a.N, a.K, a.E, a.n_in_rows, a.n_out_rows = _abi.AMOE_BF16, 16, 8, 16, 2, 8, 16
+    one = torch.zeros(64)
+    for f in ("x", "w", "out", "offsets", "in_index", "ir"):
+        setattr(a, f, one.data_ptr())
+    a.ldx, a.ldo, a.w_stride_e, a.w_stride_k, a.w_stride_n = 16, 8, 128, 8, 1
+    _abi.set_bounds(a, [0, 16])
+    a.inp_res = 1.0 / 511
+    assert ops.get_lib().amoe_cvmm_fwd(a, None) == _abi.AMOE_EUNSUPPORTED
+
+
+def test_input_gradient_with_x_but_nothing_that_reads_it(emu_ops):
+    """A caller may pass the forward input without an input range, a ReLU mask or a clipped-input output; the
+    library asks for xf_index only with one of those, so such a launch must not read through it."""
+    pr = util.make_problem(3, T=70, D=256, E=3, F=256, k=2, dtype=torch.bfloat16)
+    s_sorted, perm, in_index, offsets = emu_ops.prepare_sel(pr["idx"], 3, 2)
+    g = torch.randn(140, 256).bfloat16()
+    plain, _ = emu_ops.cvmm_bwd_x(g, pr["keys"], offsets, perm, perm, 140)
+    with_x, _ = emu_ops.cvmm_bwd_x(g, pr["keys"], offsets, perm, perm, 140, x=pr["x"])
+    assert torch.equal(plain, with_x)
 
 
 def test_argument_errors(emu_ops):

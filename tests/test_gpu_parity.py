@@ -46,7 +46,8 @@ def test_prepare_sel_bit_exact(ops, M, E, k, skew):
 
 
 def _run_case(ops, pk, lk, dtype, seed=7, routing="router", by_expert=False):
-    lk = dict(lk, by_expert=by_expert)
+    lk = dict(lk)
+    lk.setdefault("by_expert", by_expert)
     tdt = util.TORCH_DTYPE[dtype]
     pr = util.make_problem(seed, dtype=tdt, routing=routing, **pk)
     E, k, T, D, F = pk["E"], pk["k"], pk["T"], pk["D"], pk["F"]
