@@ -6,6 +6,7 @@
 #include "gemm_rows.h"
 #include "gemm_fwd256.h"
 #include "gemm_bwdx256.h"
+#include "gemm_ws256.h"
 #include "gemm_wgrad256.h"
 #include "gemm_wgrad.h"
 #include "misc_kernels.h"
@@ -140,9 +141,33 @@ int launch_bwdx256_cols(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, 
   return launch_rc();
 }
 
+// The kernel that keeps the weights in registers (gemm_ws256.h): a contraction of exactly 256, output columns in
+// groups of 256, interior launches.  Two workgroups per CU, in equal shares per column group, and more if a
+// workgroup's run of 32-row blocks would not fit its descriptor table; returns the grid, or 0 when the launch is not
+// one of these.
+inline int ws256_plan(RowsParams& p, int64_t out_rows, int64_t out_row_bytes) {
+  if (p.KD != kWsK || p.ND % 256 || !p.a_vec || !p.w_vec || !p.buf_ok || p.abs_max != nullptr) return 0;
+  if (out_rows * out_row_bytes >= (int64_t)kWsOutLimit || (int64_t)p.M * 4 >= (1LL << 31)) return 0;
+  p.n_col_blocks = p.ND / 256;
+  const long long blocks = (long long)p.M / kWsRows + p.E;                 // bound on the 32-row blocks
+  long long runs = 2LL * num_compute_units() / p.n_col_blocks;
+  if (runs < 1) runs = 1;
+  if (runs * kMaxDesc < blocks) runs = (blocks + kMaxDesc - 1) / kMaxDesc;
+  if (runs > blocks) runs = blocks;
+  return (int)(runs * p.n_col_blocks);
+}
+
 template <typename T>
 int launch_bwdx256(RowsParams p, const amoe_bwd_x_args* a, hipStream_t st, int* n_count_blocks, int* block_cols) {
   if (!rows_all_interior(p, MODE_BWDX, kFBK)) return AMOE_EUNSUPPORTED;
+  if (!bwdx_reads_x(a) && a->ir == nullptr && a->gate == nullptr && p.out_stage) {
+    // a plain product with a contraction of 256: the weights stay in registers and the rows stream past them
+    RowsParams q = p;
+    if (const int grid = ws256_plan(q, a->M, a->ldo * 2)) {
+      hipLaunchKernelGGL((&ws256_kernel<T, true, 64, WS_PLAIN, false>), dim3(grid), dim3(kThreads), 0, st, q);
+      return launch_rc();
+    }
+  }
   if (a->ir != nullptr && !a->ir_by_expert) return AMOE_EUNSUPPORTED;
   if (a->x != nullptr && (!aligned(a->x, 16) || a->ldx % 8)) return AMOE_EUNSUPPORTED;   // 16-byte pieces of x rows
   // With a short contraction an item is mostly its mask stage: 128-column tiles at three workgroups per CU then
@@ -169,16 +194,33 @@ int launch_fwd256(RowsParams p, int mode, const amoe_fwd_args* a, hipStream_t st
   // the two-K-tile variant parks the first tile's ADC codes as bytes (code + 128): a finer output quantiser than
   // 254 states does not fit them, and the general kernel (fp32 partial results) serves the launch
   if (a->n_tiles == 2 && !(p.out_half_states <= 127.f)) return AMOE_EUNSUPPORTED;
+  if (a->code_out && !analog) return AMOE_EUNSUPPORTED;
+  if (a->code_out && (!amoe_fwd_codes_supported(a) || !aligned(a->code_out, 16))) return AMOE_EUNSUPPORTED;
+  if (a->n_tiles == 1 && !a->relu && !a->xq_out && (a->x_is_quantized || !dac) && (a->code_out || !analog)) {
+    // one K-tile of 256, the operand plain or already coded, the result plain, rescaled or as ADC codes: the
+    // weights stay in registers and the rows stream past them
+    RowsParams q = p;
+    const int grid = a->code_out ? ws256_plan(q, a->n_out_rows, a->ldcode) : ws256_plan(q, a->n_out_rows, a->ldo * 2);
+    if (grid > 0) {
+      if (a->code_out) {
+        if (noisy) hipLaunchKernelGGL((&ws256_kernel<T, false, 64, WS_ZCODES, true>), dim3(grid), dim3(kThreads), 0, st, q);
+        else hipLaunchKernelGGL((&ws256_kernel<T, false, 64, WS_ZCODES, false>), dim3(grid), dim3(kThreads), 0, st, q);
+      } else if (dac) {
+        hipLaunchKernelGGL((&ws256_kernel<T, false, 64, WS_SCALE, false>), dim3(grid), dim3(kThreads), 0, st, q);
+      } else {
+        hipLaunchKernelGGL((&ws256_kernel<T, false, 64, WS_PLAIN, false>), dim3(grid), dim3(kThreads), 0, st, q);
+      }
+      return launch_rc();
+    }
+  }
   p.n_col_blocks = a->N / kFCols;
   const int grid = persistent_grid(max_row_tiles(a->M, a->E), p.n_col_blocks);
-  if (a->code_out && !analog) return AMOE_EUNSUPPORTED;
   if (!dac) return launch_fwd256_as<T, FA_PLAIN, false, false, false>(p, grid, st);
   if (!analog)
     return a->x_is_quantized ? launch_fwd256_as<T, FA_CODES, false, false, false>(p, grid, st)
                              : launch_fwd256_as<T, FA_DAC, false, false, false>(p, grid, st);
   if (a->code_out) {
     // codes leave instead of values: one output quantiser whose half range fits a byte, no second output
-    if (!amoe_fwd_codes_supported(a) || !aligned(a->code_out, 16)) return AMOE_EUNSUPPORTED;
     if (a->x_is_quantized)
       return noisy ? launch_fwd256_as<T, FA_CODES, true, true, false, true>(p, grid, st)
                    : launch_fwd256_as<T, FA_CODES, true, false, false, true>(p, grid, st);

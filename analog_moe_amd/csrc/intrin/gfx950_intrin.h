@@ -68,6 +68,21 @@ __device__ __forceinline__ BufRsrc make_rsrc(const void* base) {
 __device__ __forceinline__ u32x4 buffer_load_b128(BufRsrc r, uint32_t lane_off, uint32_t uniform_off) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0);
 }
+__device__ __forceinline__ uint32_t buffer_load_b32(BufRsrc r, uint32_t lane_off) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, 0, 0);
+}
+// Resource over [base, base + bytes): an access at a byte offset >= bytes is out of range; out-of-range stores are
+// dropped by the hardware, which makes a store conditional without a branch around it.
+__device__ __forceinline__ BufRsrc make_rsrc_sized(void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)bytes, 0x00020000);
+}
+// 16-byte store with the non-temporal hint (the data is not read again by this launch)
+__device__ __forceinline__ void buffer_store_b128_nt(BufRsrc r, u32x4 v, uint32_t lane_off) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, 0, 2);
+}
+
+// Nothing is scheduled across this point (the compiler otherwise re-orders a software pipeline to save registers).
+__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // value held by the first active lane, as a scalar
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }

@@ -13,7 +13,13 @@ def make_problem(seed, T, D, E, F, k, dtype=torch.float32, routing="router", dev
     if routing == "router":
         router = torch.randn(E, D, generator=g) / D ** 0.5
         gate, idx = torch.sigmoid(x @ router.t()).topk(k, dim=-1, sorted=False)
-    elif routing == "uniform":      # every expert gets exactly T*k/E rows
+    elif routing == "uniform":      # every expert gets exactly T*k/E rows (T*k a multiple of E), in shuffled order
+        # flat position r of the k-head list goes to expert r % E: a token's k experts are consecutive, hence
+        # distinct for k <= E; the tokens are then shuffled, which keeps every expert's count
+        base = (torch.arange(T * k) % E).reshape(T, k)
+        idx = base[torch.randperm(T, generator=g)]
+        gate = torch.rand(T, k, generator=g) * 0.5 + 0.25
+    elif routing == "near_uniform":  # k consecutive experts from a random start per token: counts T*k/E +- a few percent
         base = (torch.arange(T * k) % E).reshape(T, k)
         shift = torch.randint(0, E, (T, 1), generator=g)
         idx = (base + shift) % E

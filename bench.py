@@ -29,6 +29,11 @@ CONFIGS = {
                    name="config2: d_model=412 E=16 F=128 k=4 8192 tokens fp32"),
     "c3": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="bf16", routing="uniform", mis=512, noise=0.04,
                name="config3: d_model=1024 (2x512 tiles) E=64 F=256 k=8 16384 tokens bf16 uniform routing"),
+    # the same layer when the experts' loads differ by a few percent (k consecutive experts from a random start per
+    # token: 2048 +- 5 % rows per expert), as a router produces them: a check on the work split, not a headline
+    "c3_near": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="bf16", routing="near_uniform", mis=512, noise=0.04,
+                    name="config3 with near-uniform routing (2048 +- 5 % rows per expert): d_model=1024 (2x512 tiles) "
+                         "E=64 F=256 k=8 16384 tokens bf16"),
     "c3_f16": dict(T=16384, D=1024, E=64, F=256, k=8, dtype="f16", routing="uniform", mis=512, noise=0.04,
                    name="config3 in fp16 (the reference's reduced-precision type): d_model=1024 (2x512 tiles) E=64 "
                         "F=256 k=8 16384 tokens uniform routing"),

@@ -11,13 +11,25 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
-typedef const unsigned char* BufRsrc;
-inline BufRsrc make_rsrc(const void* base) { return static_cast<const unsigned char*>(base); }
+struct BufRsrc { const unsigned char* base; uint32_t bytes; };
+inline BufRsrc make_rsrc(const void* base) { return BufRsrc{static_cast<const unsigned char*>(base), 0xffffffffu}; }
+inline BufRsrc make_rsrc_sized(void* base, uint32_t bytes) { return BufRsrc{static_cast<const unsigned char*>(base), bytes}; }
 inline u32x4 buffer_load_b128(BufRsrc r, uint32_t lane_off, uint32_t uniform_off) {
   u32x4 v;
-  std::memcpy(&v, r + (size_t)lane_off + (size_t)uniform_off, 16);
+  std::memcpy(&v, r.base + (size_t)lane_off + (size_t)uniform_off, 16);
   return v;
 }
+inline uint32_t buffer_load_b32(BufRsrc r, uint32_t lane_off) {
+  uint32_t v;
+  std::memcpy(&v, r.base + (size_t)lane_off, 4);
+  return v;
+}
+// out-of-range stores are dropped, as the hardware's range check does
+inline void buffer_store_b128_nt(BufRsrc r, u32x4 v, uint32_t lane_off) {
+  if ((uint64_t)lane_off + 16 <= r.bytes) std::memcpy(const_cast<unsigned char*>(r.base) + lane_off, &v, 16);
+}
+// scheduling fences mean nothing to a host compiler
+inline void sched_fence() {}
 
 inline int lane_id() { return threadIdx.x & 63; }
 

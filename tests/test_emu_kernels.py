@@ -184,6 +184,11 @@ def test_result_as_adc_codes(emu_ops, noisy):
     util.check_result_as_codes(emu_ops, noisy=noisy, T=71)
 
 
+@pytest.mark.parametrize("dtype,noisy", [(torch.bfloat16, True), (torch.bfloat16, False), (torch.float16, True)])
+def test_weights_in_registers_kernel(emu_ops, dtype, noisy):
+    util.check_weights_in_registers_kernel(emu_ops, dtype=dtype, noisy=noisy)
+
+
 def test_companions(emu_ops):
     pr = util.make_problem(11, T=30, D=70, E=5, F=20, k=2)
     x = pr["x"]

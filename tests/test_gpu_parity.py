@@ -118,6 +118,15 @@ def test_wide_tiles_layer(ops, dtype):
     print(errs)
 
 
+@pytest.mark.parametrize("dtype,noisy,T,E,D", [(torch.bfloat16, True, 330, 4, 512), (torch.bfloat16, False, 9000, 9, 1024),
+                                               (torch.float16, True, 3000, 5, 256)])
+def test_weights_in_registers_kernel(ops, dtype, noisy, T, E, D):
+    """contraction of 256: the down-projection's forward (as ADC codes, rescaled, plain) and the up-projection's
+    input gradient on the kernel that holds the expert's weights in registers"""
+    print("weights in registers", dtype, noisy, T, E, D, flush=True)
+    print(util.check_weights_in_registers_kernel(ops, device="cuda", dtype=dtype, noisy=noisy, T=T, E=E, D=D))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_wide_kernels_with_uneven_experts(ops, dtype):
     print("wide kernels, uneven experts", dtype, flush=True)

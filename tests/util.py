@@ -534,3 +534,58 @@ def check_select(ops, dtype=torch.float32, device="cpu", T=70, E=24, k=3, seed=0
         want = SO.select_bwd(np32(logits), idx.cpu().numpy(), np32(gv) if use_val else None,
                              0.7 if use_reg else None, name)
         np.testing.assert_allclose(np32(got), want, **tol)
+
+
+def check_weights_in_registers_kernel(ops, device="cpu", dtype=torch.bfloat16, T=330, D=512, E=4, k=2, noisy=True):
+    """The kernel that keeps an expert's weights in registers (contraction of exactly 256): every variant against
+    the oracle, and the byte-coded result bit for bit against the 128 x 256 kernel's value result.  Uneven experts:
+    one without rows, one with more rows than a work item takes, the others ending inside a 32-row block."""
+    F = 256
+    name = dtype_name(dtype)
+    tol = {torch.bfloat16: 2e-2, torch.float16: 2e-3}[dtype]
+    g = torch.Generator().manual_seed(41)
+    idx = torch.randint(0, E - 1, (T, k), generator=g)           # expert E - 1 gets nothing
+    idx[: T // 2, 0] = 0                                         # expert 0 gets more than 256 rows
+    M = T * k
+    res = 1.0 / 127.0
+    ir = torch.linspace(0.7, 1.6, E).reshape(E, 1)
+    codes_in = torch.randint(-127, 128, (M, F), generator=g).float()
+    values = (torch.randn(E, F, D, generator=g) / F ** 0.5).to(dtype)
+    ss, perm, in_index, offsets = ops.prepare_sel(idx.to(device), E, k)
+    counts = torch.bincount(idx.reshape(-1), minlength=E)
+    assert int(counts[E - 1]) == 0 and int(counts[0]) > 256 and any(int(c) % 32 for c in counts)
+    sel_np, perm_np = ss.cpu().numpy(), perm.cpu().numpy()
+    ir_rows = ir.numpy()[sel_np]                                 # per sorted position
+    # the values whose DAC codes codes_in are: row r of the operand belongs to the expert of flat position r
+    e_of_row = idx.reshape(-1).numpy()
+    x_real = (codes_in.numpy() * np.float32(res)).astype(np.float32) * ir.numpy()[e_of_row]
+    wmax = ops.weight_abs_max(values.to(device), False)
+    wm_np = values.float().abs().amax((1, 2)).reshape(E, 1).numpy()
+    p1q, vals = codes_in.to(dtype).to(device), values.to(device)
+    common = dict(ir=ir.to(device), ir_by_expert=True, inp_res=res, x_is_quantized=True)
+    analog = dict(out_bound=12.0, out_res=254.0, wmax=wmax, noise_std=0.04 if noisy else 0.0, noise_seed=91)
+    okw = dict(inp_res=res, ir=ir_rows, dtype=name)
+    # (1) result as ADC codes (weights in registers) == result as values (128 x 256 kernel), and both against the oracle
+    codes, scale = ops.cvmm_fwd(p1q, vals, ss, offsets, perm, None, M, want_codes=True, **common, **analog)
+    z = ops.cvmm_fwd(p1q, vals, ss, offsets, perm, None, M, **common, **analog)
+    zf = ops.dequant_codes(codes, scale, idx.to(device))
+    assert torch.equal(zf.to(dtype), z)
+    want = O.cvmm_fwd(x_real, perm_np, sel_np, np32(values), out_index=None, wmax=wm_np, out_bound=12.0, out_res=254.0,
+                      noise_std=0.04 if noisy else 0.0, noise_seed=91 if noisy else None, **okw)
+    step = 12.0 * float(wm_np.max()) / 127.0 * float(ir.max())
+    flipped = adc_flip_check(np32(zf.to(dtype)), want, tol, step)
+    # (2) codes in, no output stage: the rescaled product
+    s_got = ops.cvmm_fwd(p1q, vals, ss, offsets, perm, None, M, **common)
+    s_want = O.cvmm_fwd(x_real, perm_np, sel_np, np32(values), out_index=None, **okw)
+    assert rel_err(np32(s_got), s_want) < tol
+    # (3) the plain product, column-contiguous weights (a forward) and contraction-contiguous weights (an input gradient)
+    a = torch.randn(M, F, generator=g).to(dtype)
+    p_got = ops.cvmm_fwd(a.to(device), vals, ss, offsets, perm, None, M)
+    p_want = O.cvmm_fwd(np32(a), perm_np, sel_np, np32(values), out_index=None, dtype=name)
+    assert rel_err(np32(p_got), p_want) < tol
+    keys = values.transpose(1, 2).contiguous()                  # [E, D, F]: the up-projection's weights
+    g_got, none = ops.cvmm_bwd_x(a.to(device), keys.to(device), offsets, perm, perm, M)
+    assert none is None
+    assert rel_err(np32(g_got), p_want) < tol                    # G = a @ keys[e]^T is the same product
+    assert torch.equal(g_got, p_got)
+    return dict(flipped=flipped)
