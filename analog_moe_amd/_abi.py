@@ -99,6 +99,7 @@ PROTOTYPES = {
     "amoe_row_abs_max": (C.c_int, [I32, P, I64, I64, I32, P, P]),
     "amoe_weight_abs_max": (C.c_int, [I32, P, I32, I32, I32, I32, P, P]),
     "amoe_weight_abs_max_pair": (C.c_int, [I32, P, I32, I32, P, P, I32, I32, P, I32, P]),
+    "amoe_layer_tables": (C.c_int, [I32, P, I32, I32, P, P, I32, I32, P, I32, I32, P, I32, I32, P, I32, P, P]),
     "amoe_segment_sum": (C.c_int, [P, P, I32, I32, P, I64, P]),
     "amoe_expert_std": (C.c_int, [I32, P, I64, I32, P, P, I32, P, P]),
     "amoe_modify_weight": (C.c_int, [I32, P, I32, I32, I32, P, I32, F32, F32, P, I32, C.c_uint64, P, P, P]),

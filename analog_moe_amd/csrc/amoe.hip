@@ -287,6 +287,11 @@ int amoe_prepare_sel(const void* sel, int32_t sel_is_i64, int64_t M, int32_t E, 
     hipLaunchKernelGGL(sel_hist_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
     if (int rc = launch_rc()) return rc;
   }
+  if (blocks > 0 && E <= kThreads && (long long)p.n_units * E <= kSelFuseMax && aligned(workspace, 16)) {
+    // a small table of unit counts: every workgroup of the scatter pass scans it for itself
+    hipLaunchKernelGGL(sel_scan_scatter_kernel, dim3(blocks), dim3(kThreads), 0, st, p);
+    return launch_rc();
+  }
   hipLaunchKernelGGL(sel_unit_scan_kernel, dim3((E + 3) / 4), dim3(kThreads), 0, st, p);
   if (int rc = launch_rc()) return rc;
   hipLaunchKernelGGL(sel_offsets_kernel, dim3(1), dim3(kThreads), 0, st, p);
@@ -895,19 +900,46 @@ static ColSplit col_split(int dtype, int E, int K, int N) {
 
 int amoe_weight_abs_max_pair(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a,
                              const void* w_b, int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, void* stream) {
+  return amoe_layer_tables(dtype, w_a, K_a, N_a, wmax_a, w_b, K_b, N_b, wmax_b, E, AMOE_F32, nullptr, 0, 0, nullptr, 0,
+                           nullptr, stream);
+}
+
+int amoe_layer_tables(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a, const void* w_b,
+                      int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, int32_t ir_dtype, const void* input_range,
+                      int32_t ir_cols, int32_t n_up, float* ir_up, int32_t n_dn, float* ir_dn, void* stream) {
   if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (E < 1 || K_a < 1 || N_a < 1 || K_b < 1 || N_b < 1) return AMOE_EINVAL;
   if (!w_a || !w_b || !wmax_a || !wmax_b) return AMOE_ENULL;
   if (!aligned(w_a, esize(dtype)) || !aligned(w_b, esize(dtype)) || !aligned(wmax_a, 4) || !aligned(wmax_b, 4))
     return AMOE_EALIGN;
+  if (input_range != nullptr) {
+    if (ir_dtype != AMOE_F32 && ir_dtype != AMOE_BF16 && ir_dtype != AMOE_F16) return AMOE_EINVAL;
+    if (n_up < 1 || n_dn < 1 || n_up > ir_cols || n_dn > ir_cols || ir_cols > AMOE_MAX_TILES) return AMOE_EINVAL;
+    if (!ir_up || !ir_dn) return AMOE_ENULL;
+    if (!aligned(input_range, esize(ir_dtype)) || !aligned(ir_up, 4) || !aligned(ir_dn, 4)) return AMOE_EALIGN;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const long long per_a = (long long)K_a * N_a, per_b = (long long)K_b * N_b;
   const long long per = per_a > per_b ? per_a : per_b;
   int chunks = (int)((per + 32 * kThreads - 1) / (32 * kThreads));
   chunks = chunks < 1 ? 1 : (chunks > 64 ? 64 : chunks);
   const int vec_a = aligned(w_a, 16) && (per_a % 16 == 0), vec_b = aligned(w_b, 16) && (per_b % 16 == 0);
-  hipLaunchKernelGGL(fill_zero2_kernel, dim3((E + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
-                     reinterpret_cast<uint32_t*>(wmax_a), (int)E, reinterpret_cast<uint32_t*>(wmax_b), (int)E);
+  {
+    // one small launch: the zero fill the reduction's atomic maxima start from, and the input-range tables
+    const int most = input_range ? E * (n_up > n_dn ? n_up : n_dn) : E;
+    const dim3 pg((most + kThreads - 1) / kThreads);
+    uint32_t* za = reinterpret_cast<uint32_t*>(wmax_a);
+    uint32_t* zb = reinterpret_cast<uint32_t*>(wmax_b);
+    if (ir_dtype == AMOE_F32 || input_range == nullptr)
+      hipLaunchKernelGGL((&layer_tables_prep_kernel<float>), pg, dim3(kThreads), 0, st, za, zb, (int)E,
+                         static_cast<const float*>(input_range), (int)ir_cols, (int)n_up, ir_up, (int)n_dn, ir_dn);
+    else if (ir_dtype == AMOE_BF16)
+      hipLaunchKernelGGL((&layer_tables_prep_kernel<uint16_t>), pg, dim3(kThreads), 0, st, za, zb, (int)E,
+                         static_cast<const uint16_t*>(input_range), (int)ir_cols, (int)n_up, ir_up, (int)n_dn, ir_dn);
+    else
+      hipLaunchKernelGGL((&layer_tables_prep_kernel<f16_t>), pg, dim3(kThreads), 0, st, za, zb, (int)E,
+                         static_cast<const f16_t*>(input_range), (int)ir_cols, (int)n_up, ir_up, (int)n_dn, ir_dn);
+  }
   if (int rc = launch_rc()) return rc;
   const dim3 grid(chunks, E, 2);
   if (dtype == AMOE_F32) {

@@ -374,6 +374,20 @@ __global__ __launch_bounds__(kThreads) void fill_zero2_kernel(uint32_t* __restri
   if (i < na) a[i] = 0u;
   if (i < nb) b[i] = 0u;
 }
+// fill_zero2_kernel that also makes the two fp32 input-range tables of a layer from its parameter
+// ir [2, E, ir_cols] of element type T: ir_up [E, n_up] = ir[0, :, :n_up], ir_dn [E, n_dn] = ir[1, :, :n_dn].
+template <typename T>
+__global__ __launch_bounds__(kThreads) void layer_tables_prep_kernel(uint32_t* __restrict__ a, uint32_t* __restrict__ b, int E,
+                                                                      const T* __restrict__ ir, int ir_cols, int n_up,
+                                                                      float* __restrict__ ir_up, int n_dn,
+                                                                      float* __restrict__ ir_dn) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < E) { a[i] = 0u; b[i] = 0u; }
+  if (ir != nullptr) {
+    if (i < E * n_up) ir_up[i] = Elem<T>::to_f32(ir[(long long)(i / n_up) * ir_cols + i % n_up]);
+    if (i < E * n_dn) ir_dn[i] = Elem<T>::to_f32(ir[(long long)(E + i / n_dn) * ir_cols + i % n_dn]);
+  }
+}
 // (blockIdx.z picks one of two weight tensors of the same expert count: both tables of a layer from one launch)
 template <typename T>
 __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __restrict__ w, long long per_expert,

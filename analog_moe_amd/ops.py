@@ -325,6 +325,20 @@ def weight_abs_max_pair(w_a: torch.Tensor, w_b: torch.Tensor):
     return both[0], both[1]
 
 
+def layer_tables(w_a: torch.Tensor, w_b: torch.Tensor, input_range: torch.Tensor, n_up: int, n_dn: int):
+    """``weight_abs_max_pair`` and the fp32 input-range tables of the two projections (input_range [2, E, tiles] ->
+    [E, n_up], [E, n_dn]) from the same two launches.  Returns (wmax_a, wmax_b, ir_up, ir_dn)."""
+    _need_gpu(w_a, w_b, input_range)
+    a, b = w_a.detach().contiguous(), w_b.detach().contiguous()
+    E = a.shape[0]
+    ir = input_range.detach().contiguous()
+    both = torch.empty((2, E, 1), dtype=torch.float32, device=a.device)
+    ir_up = torch.empty((E, n_up), dtype=torch.float32, device=a.device)
+    ir_dn = torch.empty((E, n_dn), dtype=torch.float32, device=a.device)
+    raw.layer_tables(get_lib(), _stream(a), a, b, both[0], both[1], ir, n_up, n_dn, ir_up, ir_dn)
+    return both[0], both[1], ir_up, ir_dn
+
+
 def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[e, t] = sum of v[i, t] over expert e's sorted rows.  ``out``: fp32 [E, columns of v] to write into (its

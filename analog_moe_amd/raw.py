@@ -291,6 +291,22 @@ def weight_abs_max_pair(lib, stream, w_a, w_b, out_a, out_b):
                                             _p(_f32(out_b, "wmax_b")), E, stream), "amoe_weight_abs_max_pair")
 
 
+def layer_tables(lib, stream, w_a, w_b, out_a, out_b, input_range, n_up: int, n_dn: int, ir_up, ir_dn):
+    """input_range [2, E, ir_cols] (any of the three dtypes, contiguous) -> ir_up fp32 [E, n_up], ir_dn fp32 [E, n_dn]"""
+    if not w_a.is_contiguous() or not w_b.is_contiguous() or w_a.dtype != w_b.dtype or w_a.shape[0] != w_b.shape[0]:
+        raise ValueError("two contiguous weight tensors of one dtype and one expert count")
+    E = w_a.shape[0]
+    if not input_range.is_contiguous() or input_range.numel() % (2 * E):
+        raise ValueError("input_range must be contiguous [2, E, tiles]")
+    ir_cols = input_range.numel() // (2 * E)
+    if tuple(ir_up.shape) != (E, n_up) or tuple(ir_dn.shape) != (E, n_dn) or not ir_up.is_contiguous() or not ir_dn.is_contiguous():
+        raise ValueError("ir_up / ir_dn must be contiguous [E, tiles of the projection]")
+    check(lib, lib.amoe_layer_tables(dtype_code(w_a), _p(w_a), w_a.shape[1], w_a.shape[2], _p(_f32(out_a, "wmax_a")),
+                                     _p(w_b), w_b.shape[1], w_b.shape[2], _p(_f32(out_b, "wmax_b")), E,
+                                     dtype_code(input_range), _p(input_range), ir_cols, n_up, _p(_f32(ir_up, "ir_up")),
+                                     n_dn, _p(_f32(ir_dn, "ir_dn")), stream), "amoe_layer_tables")
+
+
 def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out):
     """out: fp32 [E, n_tiles], rows any stride apart (a slice of a wider table will do)"""
     if (out.dtype != torch.float32 or out.dim() != 2 or tuple(out.shape) != (E, n_tiles) or

@@ -299,6 +299,15 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
 /* Both per-expert tables of a layer, wmax_a[e] = max |w_a[e]| and wmax_b[e] = max |w_b[e]| (the cols == 1 case of
  * amoe_weight_abs_max for keys [E, K_a, N_a] and values [E, K_b, N_b]), from one zero fill and one reduction
  * launch instead of two of each (moe_layer_aihwkit_lightning.py:480-487, once per projection there). */
+/* The per-expert tables one layer's forward needs, from one small launch and one reduction launch: the two max |W|
+ * tables of amoe_weight_abs_max_pair and -- with input_range != NULL -- the fp32 input-range tables of the two
+ * projections, cut out of the layer's parameter input_range [2, E, ir_cols] (element type ir_dtype):
+ * ir_up [E, n_up] = input_range[0, :, :n_up], ir_dn [E, n_dn] = input_range[1, :, :n_dn].  The reference reads that
+ * parameter through input_range[ir_idx][sel_indices.sel] once per projection and call
+ * (moe_layer_aihwkit_lightning.py:447-448); the kernels here take the table itself (ir_by_expert). */
+int amoe_layer_tables(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a, const void* w_b,
+                      int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, int32_t ir_dtype, const void* input_range,
+                      int32_t ir_cols, int32_t n_up, float* ir_up, int32_t n_dn, float* ir_dn, void* stream);
 int amoe_weight_abs_max_pair(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a,
                              const void* w_b, int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, void* stream);
 /* out[e * ldout + t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]

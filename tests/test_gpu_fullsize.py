@@ -244,6 +244,66 @@ def test_full_size_analog_layer(ops, name, T, D, E, F, k, routing, mis):
     print("input and input-range gradients ok", flush=True)
 
 
+@pytest.mark.parametrize("routing", ["uniform", "near_uniform"])
+def test_config3_full_size_generated_noise(ops, routing):
+    """The instantiations the benchmark times, at the benchmark's size: configuration 3 with the output noise DRAWN
+    IN THE KERNELS (the two-K-tile up-projection with the second output; the down-projection on the kernel that
+    holds the weights in registers, its result as ADC codes), sampled rows against float64 with the oracle's
+    counter noise.  near_uniform: expert loads that differ by a few percent, so that row tiles and block runs end
+    inside experts."""
+    from analog_moe_amd import ffn
+    from oracle import cvmm_oracle as O
+    T, D, E, F, k, mis = 16384, 1024, 64, 256, 8, 512
+    print("config3 full size, generated noise", routing, flush=True)
+    dev = "cuda"
+    pr = util.make_problem(0, T, D, E, F, k, dtype=torch.bfloat16, routing=routing)
+    pr = {n: t.to(dev) for n, t in pr.items()}
+    x, keys, values, idx, gate = (pr[n] for n in ("x", "keys", "values", "idx", "gate"))
+    M = T * k
+    bu, bd = _bounds(D, mis), _bounds(F, mis)
+    ntu, ntd = len(bu) - 1, len(bd) - 1
+    g = torch.Generator(device=dev).manual_seed(11)
+    ir = torch.empty(2, E, max(ntu, ntd), device=dev).uniform_(1.6, 2.6, generator=g)
+    ir[1] *= 0.5
+    wmax_up = keys.float().abs().amax((1, 2)).reshape(E, 1)
+    wmax_dn = values.float().abs().amax((1, 2)).reshape(E, 1)
+    seed = 0x0123456789ABCDE
+    word = torch.tensor([5], dtype=torch.int64, device=dev)          # the device part of the seed
+    cfg = ffn.FFNConfig(inp_res=RES, bounds_up=bu, bounds_down=None, out_bound=OUT_BOUND, out_res=OUT_RES,
+                        noise_std=NOISE, noise_seed=seed, noise_seed_dev=word)
+    y, p1, z, perm, in_index, offsets, z_scale, ir_up, ir_dn = ffn.ffn_forward(x, keys, values, ir, gate, idx, cfg)
+    torch.cuda.synchronize()
+    assert z.dtype == torch.uint8, "the benchmark's down-projection leaves ADC codes"
+    z = ops.dequant_codes(z, z_scale, idx)
+    flat = idx.reshape(-1)
+    ss = flat[perm.long()]
+    cpu_g = torch.Generator().manual_seed(2)
+    pos = torch.randint(0, M, (192,), generator=cpu_g)
+    pos[:8] = torch.tensor([0, 1, 31, 32, M - 1, M - 32, M // 2, M // 2 + 33])
+    pos = pos.to(dev)
+    e_of = ss[pos].long()
+    flat_pos = perm[pos].long()
+    starts = (offsets[e_of] + torch.div(pos - offsets[e_of], 32, rounding_mode="floor") * 32).cpu().numpy()
+    out_rows = flat_pos.cpu().numpy()
+
+    def drawn(n_cols, n_tiles, s, wmax_e):
+        zi = np.stack([O.counter_noise_int(out_rows, starts, n_cols, t, s) for t in range(n_tiles)]).astype(np.float64)
+        scale = ((np.float32(NOISE) * wmax_e.cpu().numpy().astype(np.float32)) * O.NOISE_SCALE).astype(np.float32)
+        return torch.from_numpy(zi * scale.astype(np.float64).reshape(1, -1, 1)).to(dev)
+
+    want_p1, step_up = _stage(x[in_index[pos].long()], keys[e_of], ir_up[e_of], bu,
+                              drawn(F, ntu, seed + 5, wmax_up[e_of]), wmax_up[e_of])
+    f1 = _flip_check(p1[flat_pos], torch.relu(want_p1), step_up, ntu, "up-projection")
+    want_z, step_dn = _stage(p1[flat_pos], values[e_of], ir_dn[e_of], bd, drawn(D, ntd, seed + 1 + 5, wmax_dn[e_of]),
+                             wmax_dn[e_of])
+    f2 = _flip_check(z[flat_pos], want_z, step_dn, ntd, "down-projection")
+    print("generated-noise samples ok; elements off by whole ADC steps:", f1, f2, flush=True)
+    # the noise is there: the same call with another device word gives another result
+    word.add_(2)
+    p1_b = ffn.ffn_forward(x, keys, values, ir, gate, idx, cfg)[1]
+    assert not torch.equal(p1_b, p1)
+
+
 @pytest.mark.parametrize("name,T,D,E,F,k,routing,mis", [("config3", 16384, 1024, 64, 256, 8, "uniform", 512)])
 def test_full_size_bf16_dac_codes_exact(ops, name, T, D, E, F, k, routing, mis):
     """Every bf16 DAC code of a full-size launch equals round((clamp(x) / r) / res) evaluated by torch in fp32 on

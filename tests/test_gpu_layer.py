@@ -58,6 +58,11 @@ def test_layer_matches_oracle(fused, split, quant):
     y.backward(dy)
     want = _oracle_for(layer, x, sel_val, sel_idx, dy, inp_res=1 / 127 if quant else -1, decay=0.01,
                        input_min_percentage=0.5, bounds_up=layer.bounds_up, bounds_down=layer.bounds_down)
+    # With the quantisers on, this END-TO-END comparison is loose on purpose: a last-bit difference in the first
+    # projection moves a few inputs of the second across a DAC rounding boundary (one step of 1/127 of the range),
+    # and those steps, not rounding error, are what 5e-3 allows.  The 1e-5 fp32 bar of the quantised path is held
+    # stage by stage, where the oracle continues from the kernel's own stage output: test_gpu_parity.py
+    # (test_layer_parity_small, test_config1_cpu_runnable_layer, test_generated_noise_interior).
     tol = 5e-3 if quant else 1e-5
     assert util.rel_err(util.np32(y).reshape(100, 128), want.y) < tol
     assert util.rel_err(util.np32(x.grad).reshape(100, 128), want.grad_x) < tol
@@ -662,6 +667,8 @@ def test_weight_abs_max_kernels():
     """moe_layer_aihwkit_lightning.py:338-344, 480-487."""
     from analog_moe_amd import ops
     util.check_weight_abs_max(ops, "cuda")
+    util.check_layer_tables(ops, "cuda")
+    util.check_layer_tables(ops, "cuda", E=64, D=1024, F=256, n_up=2, n_dn=1)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

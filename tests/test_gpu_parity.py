@@ -153,15 +153,16 @@ def test_generated_noise_matches_counter_oracle(ops):
     want = util.layer_oracle(pr, ir, "f32", backward=False,
                              wmax_up=pr["keys"].abs().amax((1, 2)).reshape(8, 1).numpy(),
                              wmax_down=pr["values"].abs().amax((1, 2)).reshape(8, 1).numpy(), **kw)
-    # hardware log / sin / cos differ from libm in the last bits
-    assert util.rel_err(got["scores"].cpu().numpy(), want.scores) < 1e-4
+    # the generator is integer arithmetic (a product of byte matrices): the kernel adds the same noise values as the
+    # oracle, so the noisy fp32 stages meet the fp32 tolerance of the noise-free path
+    assert util.rel_err(got["scores"].cpu().numpy(), want.scores) < 1e-5
     # a last-bit difference in the first stage can move an input of the second across a DAC rounding
     # boundary, so the second stage is checked from the kernel's own first-stage output
     okw = dict(wmax_up=pr["keys"].abs().amax((1, 2)).reshape(8, 1).numpy(),
                wmax_down=pr["values"].abs().amax((1, 2)).reshape(8, 1).numpy(), **kw)
     cont = util.layer_oracle(pr, ir, "f32", backward=False, got=got, **okw)
-    assert util.rel_err(got["z"].cpu().numpy(), cont.z) < 1e-4
-    assert util.rel_err(got["y"].cpu().numpy(), cont.y) < 1e-4
+    assert util.rel_err(got["z"].cpu().numpy(), cont.z) < 1e-5
+    assert util.rel_err(got["y"].cpu().numpy(), cont.y) < 1e-5
 
 
 @pytest.mark.parametrize("split", [False, True])

@@ -704,3 +704,30 @@ def test_oracle_reproduces_golden_fixture(name):
         got, ref = getattr(want, n), fx["out_" + n]
         close = np.isclose(got, ref, rtol=1e-5, atol=1e-6 * np.abs(ref).max())
         assert close.mean() > 0.999, (n, close.mean())
+
+
+def test_div_by_is_the_correctly_rounded_quotient(tmp_path):
+    """The fp32 DAC stage's "codes match exactly" rests on amoe::div_by (csrc/common.h: a / b from one multiplication
+    and two fused multiply-adds with y = 1 / b) being the IEEE quotient that torch's two divisions give
+    (cvmm.py:154, 163).  The kernels' own source is compiled for the host and compared with `/`: every one of the
+    2^23 dividend mantissas (both signs, three binades) against the 8-bit step 1/127 and three other divisors, and
+    4 x 10^7 random pairs of the DAC's operand ranges including divisors with all-ones mantissas, divisors next to a
+    power of two and the quantisation steps of 2 to 13 bits."""
+    import ctypes
+    import os
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    so = str(tmp_path / "libdivcheck.so")
+    subprocess.run(["/opt/rocm/llvm/bin/clang++", "-x", "c++", "-std=c++20", "-O2", "-fPIC", "-shared",
+                    "-ffp-contract=off", "-Wno-psabi", "-I", os.path.join(here, "emu"),
+                    "-I", os.path.join(here, "..", "include"), "-I", os.path.join(here, "..", "analog_moe_amd", "csrc"),
+                    os.path.join(here, "emu", "div_by_check.cpp"), "-o", so], check=True)
+    lib = ctypes.CDLL(so)
+    lib.div_by_mismatches_all_mantissas.restype = ctypes.c_longlong
+    lib.div_by_mismatches_all_mantissas.argtypes = [ctypes.c_float]
+    lib.div_by_mismatches_random.restype = ctypes.c_longlong
+    lib.div_by_mismatches_random.argtypes = [ctypes.c_uint64, ctypes.c_longlong, ctypes.c_int]
+    for b in (1.0 / 127.0, 2.0 / 254.0, 3.0, 1.4142135):
+        assert lib.div_by_mismatches_all_mantissas(b) == 0, b
+    for kind in range(4):
+        assert lib.div_by_mismatches_random(kind + 1, 10_000_000, kind) == 0, kind
