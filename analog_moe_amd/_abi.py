@@ -89,18 +89,18 @@ PROTOTYPES = {
     "amoe_cvmm_bwd_w": (C.c_int, [C.POINTER(BwdWArgs), P]),
     "amoe_bwd_x_workspace": (SZ, [I64, I32, I32]),
     "amoe_cvmm_bwd_x": (C.c_int, [C.POINTER(BwdXArgs), P]),
-    "amoe_gate_reduce": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
+    "amoe_gate_reduce": (C.c_int, [I32, P, P, P, I64, I32, I32, P, I64, P]),
     "amoe_ksum": (C.c_int, [I32, P, P, I64, I32, I32, P]),
     "amoe_ksum_clip_workspace": (SZ, [I64, I32, I32]),
     "amoe_ksum_clip": (C.c_int, [C.POINTER(KsumClipArgs), P]),
     "amoe_gate_grad": (C.c_int, [I32, P, P, P, I64, I32, I32, P]),
-    "amoe_gate_reduce_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),
+    "amoe_gate_reduce_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P, I64, P]),
     "amoe_gate_grad_codes": (C.c_int, [I32, P, P, P, I32, P, P, I64, I32, I32, P]),
     "amoe_row_abs_max": (C.c_int, [I32, P, I64, I64, I32, P, P]),
     "amoe_weight_abs_max": (C.c_int, [I32, P, I32, I32, I32, I32, P, P]),
     "amoe_weight_abs_max_pair": (C.c_int, [I32, P, I32, I32, P, P, I32, I32, P, I32, P]),
     "amoe_layer_tables": (C.c_int, [I32, P, I32, I32, P, P, I32, I32, P, I32, I32, P, I32, I32, P, I32, P, P]),
-    "amoe_segment_sum": (C.c_int, [P, P, I32, I32, P, I64, P]),
+    "amoe_segment_sum": (C.c_int, [P, P, I32, I32, I32, P, I64, I32, P]),
     "amoe_expert_std": (C.c_int, [I32, P, I64, I32, P, P, I32, P, P]),
     "amoe_modify_weight": (C.c_int, [I32, P, I32, I32, I32, P, I32, F32, F32, P, I32, C.c_uint64, P, P, P]),
     "amoe_weight_std_workspace": (SZ, [I32, I32, I32, I32]),

@@ -675,11 +675,16 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* a, void* stream) {
 }
 
 // ------------------------------------------------------------------------------ row-wise companions
+static int bump_only(int64_t* counter, int64_t counter_add, void* stream);
+
 static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
-                       void* stream) {
+                       void* stream, int64_t* counter_ = nullptr, int64_t counter_add_ = 0) {
   if (dtype != AMOE_F32 && dtype != AMOE_BF16 && dtype != AMOE_F16) return AMOE_EINVAL;
   if (T < 0 || k < 1 || D < 1) return AMOE_EINVAL;
-  if (T == 0) return AMOE_OK;
+  if (!aligned(counter_, 8)) return AMOE_EALIGN;
+  if (T == 0) return bump_only(counter_, counter_add_, stream);
+  long long* counter = reinterpret_cast<long long*>(counter_);
+  const long long counter_add = counter_add_;
   if (!z || !y) return AMOE_ENULL;
   const size_t es = esize(dtype);
   if (!aligned(z, es) || !aligned(y, es) || !aligned(gate, es)) return AMOE_EALIGN;
@@ -692,25 +697,35 @@ static int head_reduce(int32_t dtype, const void* z, const void* gate, void* y, 
   if (dtype == AMOE_F32) {
     auto kf = &head_reduce_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const float*>(z),
-                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D, vec);
+                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D, vec,
+                       counter, counter_add);
   } else if (dtype == AMOE_BF16) {
     auto kf = &head_reduce_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const uint16_t*>(z),
                        static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D,
-                       vec);
+                       vec, counter, counter_add);
   } else {
     auto kf = &head_reduce_kernel<f16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const f16_t*>(z),
                        static_cast<const f16_t*>(gate), static_cast<f16_t*>(y), (long long)T, (int)k, (int)D,
-                       vec);
+                       vec, counter, counter_add);
   }
   return launch_rc();
 }
 
+// the counter still moves when a call has no rows to reduce
+__global__ void bump_kernel(long long* counter, long long add) { bump_counter(counter, add); }
+static int bump_only(int64_t* counter, int64_t counter_add, void* stream) {
+  if (!counter) return AMOE_OK;
+  hipLaunchKernelGGL(bump_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<long long*>(counter), (long long)counter_add);
+  return launch_rc();
+}
+
 int amoe_gate_reduce(int32_t dtype, const void* z, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
-                     void* stream) {
+                     int64_t* counter, int64_t counter_add, void* stream) {
   if (T > 0 && !gate) return AMOE_ENULL;
-  return head_reduce(dtype, z, gate, y, T, k, D, stream);
+  return head_reduce(dtype, z, gate, y, T, k, D, stream, counter, counter_add);
 }
 
 int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, int32_t D, void* stream) {
@@ -810,24 +825,31 @@ static int codes_args_ok(int32_t dtype, const uint8_t* codes, const float* scale
 }
 
 int amoe_gate_reduce_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel, int32_t sel_is_i64,
-                           const void* gate, void* y, int64_t T, int32_t k, int32_t D, void* stream) {
+                           const void* gate, void* y, int64_t T, int32_t k, int32_t D, int64_t* counter_,
+                           int64_t counter_add_, void* stream) {
   if (int rc = codes_args_ok(dtype, codes, scale, sel, sel_is_i64, gate, y, T, k, D)) return rc;
-  if (T == 0) return AMOE_OK;
+  if (!aligned(counter_, 8)) return AMOE_EALIGN;
+  if (T == 0) return bump_only(counter_, counter_add_, stream);
+  long long* counter = reinterpret_cast<long long*>(counter_);
+  const long long counter_add = counter_add_;
   const long long blocks = ((long long)T * (D / 16) + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return AMOE_EUNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == AMOE_F32) {
     auto kf = &head_reduce_codes_kernel<float>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
-                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D);
+                       static_cast<const float*>(gate), static_cast<float*>(y), (long long)T, (int)k, (int)D,
+                       counter, counter_add);
   } else if (dtype == AMOE_BF16) {
     auto kf = &head_reduce_codes_kernel<uint16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
-                       static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D);
+                       static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(y), (long long)T, (int)k, (int)D,
+                       counter, counter_add);
   } else {
     auto kf = &head_reduce_codes_kernel<f16_t>;
     hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(kThreads), 0, st, codes, scale, sel, (int)sel_is_i64,
-                       static_cast<const f16_t*>(gate), static_cast<f16_t*>(y), (long long)T, (int)k, (int)D);
+                       static_cast<const f16_t*>(gate), static_cast<f16_t*>(y), (long long)T, (int)k, (int)D,
+                       counter, counter_add);
   }
   return launch_rc();
 }
@@ -1024,13 +1046,29 @@ int amoe_weight_abs_max(int32_t dtype, const void* w, int32_t E, int32_t K, int3
   return launch_rc();
 }
 
-int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, float* out, int64_t ldout,
-                     void* stream) {
-  if (E < 1 || n_tiles < 1 || n_tiles > AMOE_MAX_TILES || ldout < n_tiles) return AMOE_EINVAL;
+int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, int32_t out_dtype, void* out,
+                     int64_t ldout, int32_t zero_cols, void* stream) {
+  if (out_dtype != AMOE_F32 && out_dtype != AMOE_BF16 && out_dtype != AMOE_F16) return AMOE_EINVAL;
+  if (E < 1 || n_tiles < 1 || n_tiles > AMOE_MAX_TILES || zero_cols < 0 || zero_cols > AMOE_MAX_TILES ||
+      ldout < n_tiles + zero_cols)
+    return AMOE_EINVAL;
   if (!v || !offsets || !out) return AMOE_ENULL;
-  if (!aligned(v, 4) || !aligned(offsets, 4) || !aligned(out, 4)) return AMOE_EALIGN;
-  hipLaunchKernelGGL(segment_sum_kernel, dim3(E, n_tiles), dim3(kThreads), 0, static_cast<hipStream_t>(stream), v,
-                     offsets, (int)n_tiles, out, (long long)ldout);
+  if (!aligned(v, 4) || !aligned(offsets, 4) || !aligned(out, esize(out_dtype))) return AMOE_EALIGN;
+  const dim3 grid(E, n_tiles + zero_cols);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_dtype == AMOE_F32) {
+    auto kf = &segment_sum_kernel<float>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, v, offsets, (int)n_tiles, static_cast<float*>(out),
+                       (long long)ldout);
+  } else if (out_dtype == AMOE_BF16) {
+    auto kf = &segment_sum_kernel<uint16_t>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, v, offsets, (int)n_tiles, static_cast<uint16_t*>(out),
+                       (long long)ldout);
+  } else {
+    auto kf = &segment_sum_kernel<f16_t>;
+    hipLaunchKernelGGL(kf, grid, dim3(kThreads), 0, st, v, offsets, (int)n_tiles, static_cast<f16_t*>(out),
+                       (long long)ldout);
+  }
   return launch_rc();
 }
 

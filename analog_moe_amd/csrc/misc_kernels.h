@@ -6,14 +6,22 @@
 
 namespace amoe {
 
+// The step counter of the generated noise moves on in the launch that follows the last kernel drawing from it: stream
+// order puts every read of the old value before this addition (one lane, a vector-memory atomic).
+__device__ __forceinline__ void bump_counter(long long* counter, long long add) {
+  if (counter != nullptr && blockIdx.x == 0 && threadIdx.x == 0)
+    atomicAdd(reinterpret_cast<unsigned long long*>(counter), (unsigned long long)add);
+}
+
 // y[t, d] = sum_j gate[t*k+j] * z[(t*k+j), d]   (gate == nullptr: plain sum over j).
 // One thread per (row, 16-byte chunk); fp32 accumulation in ascending j.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void head_reduce_kernel(const T* __restrict__ z, const T* __restrict__ gate,
                                                                 T* __restrict__ y, long long rows, int k, int D,
-                                                                int vec) {
+                                                                int vec, long long* counter, long long counter_add) {
   constexpr int CH = Elem<T>::kChunk;
   const int chunks = (D + CH - 1) / CH;
+  bump_counter(counter, counter_add);
   const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
   if (idx >= rows * chunks) return;
   const long long t = idx / chunks;
@@ -108,8 +116,10 @@ __global__ __launch_bounds__(kThreads) void head_reduce_codes_kernel(const uint8
                                                                       const float* __restrict__ scale,
                                                                       const void* __restrict__ sel, int sel_is_i64,
                                                                       const T* __restrict__ gate, T* __restrict__ y,
-                                                                      long long rows, int k, int D) {
+                                                                      long long rows, int k, int D,
+                                                                      long long* counter, long long counter_add) {
   const int chunks = D / 16;
+  bump_counter(counter, counter_add);
   const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
   if (idx >= rows * chunks) return;
   const long long t = idx / chunks;
@@ -434,20 +444,23 @@ __global__ __launch_bounds__(kThreads) void weight_abs_max_kernel(const T* __res
   }
 }
 
-// out[e, t] = sum_{i in [offsets[e], offsets[e+1])} v[i, t], one workgroup per (expert, tile).
+// out[e, t] = sum_{i in [offsets[e], offsets[e+1])} v[i, t], one workgroup per (expert, column); columns from n_tiles
+// on (gridDim.y may exceed n_tiles) receive zero.  T: element type of out (one rounding of the fp32 sum).
+template <typename T>
 __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float* __restrict__ v,
                                                                 const int32_t* __restrict__ offsets, int n_tiles,
-                                                                float* __restrict__ out, long long ldout) {
+                                                                T* __restrict__ out, long long ldout) {
   __shared__ float red[4];
   const int e = blockIdx.x, t = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
   float s = 0.f;
-  for (int i = offsets[e] + tid; i < offsets[e + 1]; i += kThreads) s += v[(long long)i * n_tiles + t];
+  if (t < n_tiles)
+    for (int i = offsets[e] + tid; i < offsets[e + 1]; i += kThreads) s += v[(long long)i * n_tiles + t];
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) s += wave_shfl_xor(s, d);
   if (lane == 0) red[tid >> 6] = s;
   __syncthreads();
-  if (tid == 0) out[(long long)e * ldout + t] = (red[0] + red[1]) + (red[2] + red[3]);
+  if (tid == 0) out[(long long)e * ldout + t] = Elem<T>::cvt((red[0] + red[1]) + (red[2] + red[3]));
 }
 
 __device__ __forceinline__ double block_sum_double(double v, double* red /* LDS [4] */) {

@@ -35,6 +35,8 @@ class FFNConfig:
     noise_down: Optional[torch.Tensor] = None
     wmax_up: Optional[torch.Tensor] = None        # max |W| behind noise and ADC when the weights passed in are
     wmax_down: Optional[torch.Tensor] = None      # modified copies (fp32 [E, 1] or [E, N]); None: taken from them
+    seed_bump: int = 0                            # added to noise_seed_dev by the forward's last launch (eager calls
+                                                  # only: not among the fields the opaque operators take)
 
 
 _SIDE_STREAMS = {}
@@ -90,12 +92,15 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
         side = _side_stream(x.device)
         side.wait_stream(main)
         with torch.cuda.stream(side):
-            ir_up, ir_dn = ir_tables(input_range, E, cfg)
             if cfg.noise_per_channel:
+                ir_up, ir_dn = ir_tables(input_range, E, cfg)
                 wu = ops.weight_abs_max(keys, True)
                 wd = ops.weight_abs_max(values, True)
-            else:
+            elif input_range is None:
                 wu, wd = ops.weight_abs_max_pair(keys, values)
+            else:                                # both max |W| tables and both fp32 range tables from two launches
+                wu, wd, ir_up, ir_dn = ops.layer_tables(keys, values, input_range.reshape(2, E, -1),
+                                                        _n_tiles(cfg.bounds_up), _n_tiles(cfg.bounds_down))
         for t in (wu, wd, ir_up, ir_dn):
             if t is not None:
                 t.record_stream(main)
@@ -116,15 +121,17 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
     p1, p1q = p1 if chain else (p1, None)
     down = dict(ir=ir_dn, bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
                 noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
+    # the gate reduction follows the last launch that draws noise: it moves the device seed word on
+    bump = (cfg.noise_seed_dev, cfg.seed_bump) if cfg.seed_bump and cfg.noise_seed_dev is not None else ()
     if chain and z_as_codes(p1q, values, cfg):
         # the down-projection's result is read twice more and never as a matrix operand (gate reduction now, gate
         # gradient in the backward pass): it is kept as its ADC codes, one byte per value, with two factors per expert
         z, z_scale = ops.cvmm_fwd(p1q, values, sel_sorted, offsets, perm, None, M, want_codes=True, **down)
-        y = ops.gate_reduce_codes(z, z_scale, sel_idx, gate)
+        y = ops.gate_reduce_codes(z, z_scale, sel_idx, gate, *bump)
     else:
         z = ops.cvmm_fwd(p1q if chain else p1, values, sel_sorted, offsets, perm, None, M, **down)
         z_scale = torch.empty(0, dtype=torch.float32, device=x.device)
-        y = ops.gate_reduce(z, gate)
+        y = ops.gate_reduce(z, gate, *bump)
     return y, p1, z, perm, in_index, offsets, z_scale, ir_up, ir_dn
 
 
@@ -136,8 +143,8 @@ def z_as_codes(p1q: torch.Tensor, values: torch.Tensor, cfg: FFNConfig) -> bool:
 
 
 def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn,
-                 cfg: FFNConfig, want_ir_grad: bool):
-    """Returns (grad_x, grad_keys, grad_values, grad_ir [2, E, n_tiles] fp32 or None, grad_gate)."""
+                 cfg: FFNConfig, want_ir_grad: bool, ir_dtype: torch.dtype = torch.float32):
+    """Returns (grad_x, grad_keys, grad_values, grad_ir [2, E, n_tiles] of type ir_dtype or None, grad_gate)."""
     E = keys.shape[0]
     k = gate.shape[-1]
     M = perm.numel()
@@ -161,8 +168,10 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
         full, irg_up = ops.cvmm_bwd_x(gp1, keys, offsets, perm, perm, M, x=x, xf_index=in_index, ir=ir_up,
                                       bounds=cfg.bounds_up, **irkw, **by)
     # the gate gradient and the sum over the k heads only stream z, dy and the per-head input gradient
-    # through HBM; they run on a second stream next to the two weight gradients, whose workgroups
-    # leave registers and wave slots free on every CU
+    # through HBM; they run on a second stream next to the two weight gradients.  With evenly loaded experts the
+    # four launches take as long side by side as one after the other (together they are bound by memory traffic);
+    # with uneven loads the streaming kernels fill the CUs that the weight gradients' last tiles leave idle
+    # (2 - 3 % of the step)
     main, side = torch.cuda.current_stream(), _side_stream(x.device)
     side.wait_stream(main)
     with torch.cuda.stream(side):
@@ -180,17 +189,17 @@ def ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_in
     grad_ir = None
     if ir_up is not None and want_ir_grad:
         ntu, ntd = ir_up.shape[1], ir_dn.shape[1]
-        # the two tables of per-expert sums are written where they belong; only columns neither has need a zero.
-        # The fill and the down-projection's sums are issued here, where the second stream keeps the GPU busy,
-        # instead of after the join at the end of the step
-        make = torch.empty if ntu == ntd else torch.zeros
-        grad_ir = make((2, E, max(ntu, ntd)), dtype=torch.float32, device=x.device)
-        ops.segment_sum(irg_dn, offsets, E, out=grad_ir[1, :, :ntd])
+        # the two tables of per-expert sums are written where they belong, in the parameter's type, and each launch
+        # clears the columns its projection does not have.  The down-projection's sums are issued here, where the
+        # second stream keeps the GPU busy, instead of after the join at the end of the step
+        nt = max(ntu, ntd)
+        grad_ir = torch.empty((2, E, nt), dtype=ir_dtype, device=x.device)
+        ops.segment_sum(irg_dn, offsets, E, out=grad_ir[1, :, :ntd], zero_cols=nt - ntd)
     grad_values = ops.cvmm_bwd_w(p1c, dy, E, offsets, perm, tok)
     grad_keys = ops.cvmm_bwd_w(x, gp1, E, offsets, in_index, perm, ir=ir_up, bounds=cfg.bounds_up, **by)
     main.wait_stream(side)
     if grad_ir is not None:
-        ops.segment_sum(irg_up, offsets, E, out=grad_ir[0, :, :ntu])
+        ops.segment_sum(irg_up, offsets, E, out=grad_ir[0, :, :ntu], zero_cols=nt - ntu)
     return grad_x, grad_keys, grad_values, grad_ir, grad_gate
 
 
@@ -213,9 +222,9 @@ class AnalogMoEFFN(torch.autograd.Function):
         x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn = ctx.saved_tensors
         grad_x, grad_keys, grad_values, grad_ir, grad_gate = ffn_backward(
             dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets, ir_up, ir_dn, ctx.cfg,
-            ctx.needs_input_grad[3])
+            ctx.needs_input_grad[3], ctx.ir_dtype or torch.float32)
         if grad_ir is not None:
-            grad_ir = grad_ir.reshape(ctx.ir_shape).to(ctx.ir_dtype)
+            grad_ir = grad_ir.reshape(ctx.ir_shape)
         return grad_x, grad_keys, grad_values, grad_ir, grad_gate, None, None
 
 

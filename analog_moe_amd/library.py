@@ -322,11 +322,12 @@ def ffn_bwd(dy, x, keys, values, input_range, gate, sel_idx, p1, z, z_scale, per
     c = _cfg(cfg)
     ir_up, ir_dn = ffn.ir_tables(input_range, keys.shape[0], c)
     gx, gk, gv, gir, gg = ffn.ffn_backward(dy, x, keys, values, gate, sel_idx, p1, z, z_scale, perm, in_index, offsets,
-                                           ir_up, ir_dn, c, want_ir_grad)
+                                           ir_up, ir_dn, c, want_ir_grad,
+                                           torch.float32 if input_range is None else input_range.dtype)
     if gir is None:
         gir = torch.empty(_EMPTY_SHAPE, dtype=torch.float32, device=x.device)
     else:
-        gir = gir.reshape(input_range.shape).to(input_range.dtype)
+        gir = gir.reshape(input_range.shape)
     return gx, gk, gv, gir, gg
 
 

@@ -673,12 +673,17 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
             if dt not in (torch.bfloat16, torch.float16):
                 raise MoEConifgError("the CVMM kernels autocast to bfloat16 or float16")
             x = x.to(dt)
+        # the two projections use seed + 0 and seed + 1, so the device word moves by 2 per call; a weight modifier alone
+        # (no output noise) must see a new word too.  Called eagerly, the layer's last forward launch adds it; under
+        # torch.compile (opaque operators that declare no mutation) the addition stays a torch operation
+        bump_here = self.noise_counter is not None and (drew or cfg.noise_seed_dev is not None)
+        if bump_here and cfg.noise_seed_dev is not None and not torch.compiler.is_compiling():
+            cfg.seed_bump, bump_here = 2, False
         y = moe_ffn(x.reshape(-1, x.shape[-1]), keys.to(x.dtype), values.to(x.dtype),
                     self.input_range, sel_val.reshape(-1, self.n_heads).to(x.dtype),
                     sel_idx.reshape(-1, self.n_heads), cfg)
-        if self.noise_counter is not None and (drew or cfg.noise_seed_dev is not None):
-            self.noise_counter.add_(2)             # the two projections used seed + 0 and seed + 1; a weight
-                                                   # modifier alone (no output noise) must see a new word too
+        if bump_here:
+            self.noise_counter.add_(2)
         y = y.view(*lead, self.v_dim)
         if self.o_bias is not None:
             y = y + self.o_bias

@@ -205,28 +205,31 @@ def cvmm_bwd_x(g: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, g_index:
 
 
 # ------------------------------------------------------------------------------ companions
-def gate_reduce(z: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
-    """y[t] = sum_j gate[t, j] * z[t, j]; z [T*k, D] (or [..., k, D]), gate [..., k]."""
-    _need_gpu(z, gate)
+def gate_reduce(z: torch.Tensor, gate: torch.Tensor, counter: Optional[torch.Tensor] = None,
+                counter_add: int = 0) -> torch.Tensor:
+    """y[t] = sum_j gate[t, j] * z[t, j]; z [T*k, D] (or [..., k, D]), gate [..., k].  counter: an int64 device word
+    to which the same launch adds counter_add (the step counter of the generated noise)."""
+    _need_gpu(z, gate, counter)
     k = gate.shape[-1]
     z2 = _rows2d(z).contiguous()
     T, D = z2.shape[0] // k, z2.shape[1]
     gate_c = gate.detach().reshape(-1).to(z2.dtype).contiguous()
     y = torch.empty((T, D), dtype=z2.dtype, device=z2.device)
-    raw.gate_reduce(get_lib(), _stream(z2), z2, gate_c, y, T, k, D)
+    raw.gate_reduce(get_lib(), _stream(z2), z2, gate_c, y, T, k, D, counter, counter_add)
     return y
 
 
-def gate_reduce_codes(codes: torch.Tensor, scale: torch.Tensor, sel: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+def gate_reduce_codes(codes: torch.Tensor, scale: torch.Tensor, sel: torch.Tensor, gate: torch.Tensor,
+                      counter: Optional[torch.Tensor] = None, counter_add: int = 0) -> torch.Tensor:
     """``gate_reduce`` of a k-head tensor stored as ADC codes (``cvmm_fwd(..., want_codes=True)``); sel [..., k]: the
     expert of every (token, head)."""
-    _need_gpu(codes, scale, sel, gate)
+    _need_gpu(codes, scale, sel, gate, counter)
     k = gate.shape[-1]
     T, D = codes.shape[0] // k, codes.shape[1]
     gate_c = gate.detach().reshape(-1).contiguous()
     sel_c = sel.detach().reshape(-1).contiguous()
     y = torch.empty((T, D), dtype=gate_c.dtype, device=codes.device)
-    raw.gate_reduce_codes(get_lib(), _stream(codes), codes, scale, sel_c, gate_c, y, T, k, D)
+    raw.gate_reduce_codes(get_lib(), _stream(codes), codes, scale, sel_c, gate_c, y, T, k, D, counter, counter_add)
     return y
 
 
@@ -340,9 +343,10 @@ def layer_tables(w_a: torch.Tensor, w_b: torch.Tensor, input_range: torch.Tensor
 
 
 def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[e, t] = sum of v[i, t] over expert e's sorted rows.  ``out``: fp32 [E, columns of v] to write into (its
-    rows may lie further apart than its columns: a slice of a wider table)."""
+                out: Optional[torch.Tensor] = None, zero_cols: int = 0) -> torch.Tensor:
+    """out[e, t] = sum of v[i, t] over expert e's sorted rows (fp32 sums, rounded once to out's type).  ``out``:
+    [E, columns of v] to write into (its rows may lie further apart than its columns: a slice of a wider table, whose
+    next ``zero_cols`` columns are cleared by the same launch)."""
     _need_gpu(v, offsets)
     cols = 1
     for d in v.shape[1:]:
@@ -351,8 +355,10 @@ def segment_sum(v: torch.Tensor, offsets: torch.Tensor, n_experts: int,
     if out is None:
         out = torch.empty((n_experts, cols), dtype=torch.float32, device=v2.device)
     if v2.shape[0] == 0:                           # no sorted positions at all: nothing to read
+        if zero_cols:
+            out.as_strided((n_experts, zero_cols), (out.stride(0), 1), out.storage_offset() + cols).zero_()
         return out.zero_()
-    raw.segment_sum(get_lib(), _stream(v2), v2, offsets, n_experts, cols, out)
+    raw.segment_sum(get_lib(), _stream(v2), v2, offsets, n_experts, cols, out, zero_cols)
     return out
 
 

@@ -210,13 +210,23 @@ def cvmm_bwd_x(lib, stream, g, w, grad_x_full, offsets, g_index, out_index, x=No
     check(lib, lib.amoe_cvmm_bwd_x(C.byref(a), stream), "amoe_cvmm_bwd_x")
 
 
-def gate_reduce(lib, stream, z, gate, y, T: int, k: int, D: int):
-    check(lib, lib.amoe_gate_reduce(dtype_code(z), _p(z), _p(gate), _p(y), T, k, D, stream), "amoe_gate_reduce")
+def _counter(counter):
+    """An int64 device word the launch adds to (None: no addition)."""
+    if counter is not None and (counter.dtype != torch.int64 or counter.numel() < 1):
+        raise ValueError("counter must be an int64 tensor (one word in device memory)")
+    return _p(counter)
 
 
-def gate_reduce_codes(lib, stream, codes, scale, sel, gate, y, T: int, k: int, D: int):
+def gate_reduce(lib, stream, z, gate, y, T: int, k: int, D: int, counter=None, counter_add: int = 0):
+    check(lib, lib.amoe_gate_reduce(dtype_code(z), _p(z), _p(gate), _p(y), T, k, D, _counter(counter), counter_add,
+                                    stream), "amoe_gate_reduce")
+
+
+def gate_reduce_codes(lib, stream, codes, scale, sel, gate, y, T: int, k: int, D: int, counter=None,
+                      counter_add: int = 0):
     check(lib, lib.amoe_gate_reduce_codes(dtype_code(y), _p(codes), _p(scale), _p(sel), int(sel.dtype == torch.int64),
-                                          _p(gate), _p(y), T, k, D, stream), "amoe_gate_reduce_codes")
+                                          _p(gate), _p(y), T, k, D, _counter(counter), counter_add, stream),
+          "amoe_gate_reduce_codes")
 
 
 def gate_grad_codes(lib, stream, codes, scale, sel, dy, grad_gate, T: int, k: int, D: int):
@@ -307,13 +317,14 @@ def layer_tables(lib, stream, w_a, w_b, out_a, out_b, input_range, n_up: int, n_
                                      n_dn, _p(_f32(ir_dn, "ir_dn")), stream), "amoe_layer_tables")
 
 
-def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out):
-    """out: fp32 [E, n_tiles], rows any stride apart (a slice of a wider table will do)"""
-    if (out.dtype != torch.float32 or out.dim() != 2 or tuple(out.shape) != (E, n_tiles) or
-            (n_tiles > 1 and out.stride(1) != 1) or out.stride(0) < n_tiles):
-        raise ValueError("out must be float32 [E, n_tiles] with unit column stride")
-    check(lib, lib.amoe_segment_sum(_p(_f32(v, "v")), _p(_i32(offsets, "offsets")), E, n_tiles,
-                                    _p(out), out.stride(0), stream), "amoe_segment_sum")
+def segment_sum(lib, stream, v, offsets, E: int, n_tiles: int, out, zero_cols: int = 0):
+    """out: [E, n_tiles] in any of the three dtypes, rows any stride apart (a slice of a wider table will do); the
+    zero_cols columns that follow the slice in that table are cleared"""
+    if (out.dim() != 2 or tuple(out.shape) != (E, n_tiles) or (n_tiles > 1 and out.stride(1) != 1) or
+            out.stride(0) < n_tiles + zero_cols):
+        raise ValueError("out must be [E, n_tiles] with unit column stride and rows at least n_tiles + zero_cols apart")
+    check(lib, lib.amoe_segment_sum(_p(_f32(v, "v")), _p(_i32(offsets, "offsets")), E, n_tiles, dtype_code(out),
+                                    _p(out), out.stride(0), zero_cols, stream), "amoe_segment_sum")
 
 
 def expert_std(lib, stream, x, in_index, offsets, E: int, out):

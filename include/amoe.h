@@ -241,9 +241,13 @@ int amoe_cvmm_bwd_x(const amoe_bwd_x_args* args, void* stream);
 /* ---------------------------------------------------------------------------------------
  * Small row-wise companions of CVMM.forward / CVMM.backward.
  */
-/* y[t, :] = sum_j gate[t, j] * z[t*k + j, :]   (cvmm.py:757-759) */
+/* y[t, :] = sum_j gate[t, j] * z[t*k + j, :]   (cvmm.py:757-759).
+ * counter (may be NULL): an int64 word in device memory to which the launch adds counter_add.  The layer passes the
+ * step counter of the generated noise (amoe_fwd_args.noise_seed_dev): this is the launch that follows the last
+ * kernel drawing from it, so the next forward, or the next replay of a captured graph, draws anew without a launch
+ * of its own for the addition (the reference draws fresh torch.randn tensors per call, cvmm.py:712-716). */
 int amoe_gate_reduce(int32_t dtype, const void* z, const void* gate, void* y,
-                     int64_t T, int32_t k, int32_t D, void* stream);
+                     int64_t T, int32_t k, int32_t D, int64_t* counter, int64_t counter_add, void* stream);
 /* out[t, :] = sum_j full[t*k + j, :]           (cvmm.py:890-891) */
 int amoe_ksum(int32_t dtype, const void* full, void* out, int64_t T, int32_t k, int32_t D,
               void* stream);
@@ -285,7 +289,7 @@ int amoe_gate_grad(int32_t dtype, const void* z, const void* dy, void* grad_gate
  * belongs to expert sel[r] (the unsorted ids, int32 or int64), z[r, :] = ((code[r, :] - 128) * scale[e][0]) * scale[e][1]. */
 int amoe_gate_reduce_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel,
                            int32_t sel_is_i64, const void* gate, void* y, int64_t T, int32_t k, int32_t D,
-                           void* stream);
+                           int64_t* counter, int64_t counter_add, void* stream);
 int amoe_gate_grad_codes(int32_t dtype, const uint8_t* codes, const float* scale, const void* sel,
                          int32_t sel_is_i64, const void* dy, void* grad_gate, int64_t T, int32_t k, int32_t D,
                          void* stream);
@@ -311,10 +315,11 @@ int amoe_layer_tables(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, 
 int amoe_weight_abs_max_pair(int32_t dtype, const void* w_a, int32_t K_a, int32_t N_a, float* wmax_a,
                              const void* w_b, int32_t K_b, int32_t N_b, float* wmax_b, int32_t E, void* stream);
 /* out[e * ldout + t] = sum_{i in expert e} v[i, t]: index backward of input_range[sel]
- * (moe_layer_aihwkit_lightning.py:447-448), fixed order.  ldout >= n_tiles: the row stride of out, so that the
- * sums can land in a slice of a wider table. */
-int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles,
-                     float* out, int64_t ldout, void* stream);
+ * (moe_layer_aihwkit_lightning.py:447-448), fixed order, fp32 sums rounded once to out_dtype (the parameter's type).
+ * ldout >= n_tiles + zero_cols: the row stride of out, so that the sums can land in a slice of a wider table; the
+ * zero_cols columns after the sums are set to zero (tile columns of the table that this projection does not have). */
+int amoe_segment_sum(const float* v, const int32_t* offsets, int32_t E, int32_t n_tiles, int32_t out_dtype,
+                     void* out, int64_t ldout, int32_t zero_cols, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Per-expert unbiased standard deviation of the routed rows' elements, for input-range

@@ -198,6 +198,8 @@ def test_companions(emu_ops):
     util.check_weight_abs_max(emu_ops)
     util.check_layer_tables(emu_ops)
     util.check_layer_tables(emu_ops, dtype=torch.float32, E=3, n_up=1, n_dn=3)
+    util.check_segment_sum_typed(emu_ops)
+    util.check_gate_reduce_counter(emu_ops)
     va = pr["values"].to(torch.float16)[:, :, :61].contiguous()                      # 20 x 61: no 16-byte slices
     wa, wb = emu_ops.weight_abs_max_pair(pr["keys"].to(torch.float16), va)
     assert torch.equal(wb, va.float().abs().amax((1, 2)).reshape(5, 1))

@@ -671,6 +671,12 @@ def test_weight_abs_max_kernels():
     util.check_layer_tables(ops, "cuda", E=64, D=1024, F=256, n_up=2, n_dn=1)
 
 
+def test_segment_sums_in_the_parameter_type_and_counter_in_the_gate_reduction():
+    from analog_moe_amd import ops
+    util.check_segment_sum_typed(ops, "cuda")
+    util.check_gate_reduce_counter(ops, "cuda")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("per_channel", [False, True])
 def test_weight_std_and_clamp_kernels_match_oracle(per_channel, dtype):

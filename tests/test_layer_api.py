@@ -299,7 +299,7 @@ def test_library_rejects_bad_arguments_on_the_host():
     assert lib.amoe_cvmm_bwd_x(bwd_x(relu_mask=1), None) == ENULL          # a mask needs the forward input
     assert lib.amoe_cvmm_bwd_x(bwd_x(ldo=16), None) == ESHAPE
     # companions
-    assert lib.amoe_gate_reduce(_abi.AMOE_F32, p, None, p, 4, 2, 8, None) == ENULL
+    assert lib.amoe_gate_reduce(_abi.AMOE_F32, p, None, p, 4, 2, 8, None, 0, None) == ENULL
     assert lib.amoe_gate_grad(5, p, p, p, 4, 2, 8, None) == EINVAL
     assert lib.amoe_row_abs_max(_abi.AMOE_F32, p, 4, 8, 16, p, None) == EINVAL          # ldx < K
     assert lib.amoe_weight_abs_max(_abi.AMOE_F32, p, 2, 8, 16, 3, p, None) == EINVAL   # cols is 1 or N

@@ -1,6 +1,7 @@
 """Shared by the CPU (emulated) and GPU parity tests: builds seeded problems, runs the layer
 through analog_moe_amd.ops and through the oracle, and compares."""
 import numpy as np
+import pytest
 import torch
 
 from analog_moe_amd.synthetic import make_problem  # noqa: F401  (re-exported: the tests build their inputs with it)
@@ -602,3 +603,40 @@ def check_layer_tables(ops, device="cpu", dtype=torch.bfloat16, E=5, D=72, F=40,
         assert torch.equal(wu, ops.weight_abs_max(keys, False)) and torch.equal(wd, ops.weight_abs_max(values, False))
         assert torch.equal(ir_up, ir[0, :, :n_up].float()) and torch.equal(ir_dn, ir[1, :, :n_dn].float())
         assert ir_up.dtype == torch.float32 and ir_up.is_contiguous() and ir_dn.is_contiguous()
+
+
+def check_segment_sum_typed(ops, device="cpu"):
+    """Per-expert sums land in a slice of a wider table, in the table's type, and clear the columns after the slice
+    (the index backward of input_range[sel], moe_layer_aihwkit_lightning.py:447-448, sums in the parameter's type)."""
+    g = torch.Generator().manual_seed(5)
+    offsets = torch.tensor([0, 3, 3, 10, 11, 40, 57], dtype=torch.int32, device=device)      # one expert without rows
+    E = offsets.numel() - 1
+    v = torch.randn(57, 2, generator=g).to(device)
+    want = torch.stack([v[offsets[e]:offsets[e + 1]].double().sum(0) for e in range(E)])
+    plain = ops.segment_sum(v, offsets, E)
+    assert plain.dtype == torch.float32 and (plain.double() - want).abs().max() < 1e-5
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        table = torch.full((2, E, 4), 7.0, dtype=dt, device=device)
+        ops.segment_sum(v, offsets, E, out=table[1, :, :2], zero_cols=1)
+        assert torch.equal(table[1, :, :2], plain.to(dt))                    # one rounding of the fp32 sum
+        assert bool((table[1, :, 2] == 0).all()) and bool((table[1, :, 3] == 7).all()) and bool((table[0] == 7).all())
+    with pytest.raises(ValueError):
+        ops.segment_sum(v, offsets, E, out=torch.zeros(E, 2, device=device), zero_cols=1)     # rows too close
+
+
+def check_gate_reduce_counter(ops, device="cpu"):
+    """The gate reductions add to a device word in the same launch (the step counter of the generated noise), also
+    when there is nothing to reduce; the reduction itself is unchanged."""
+    g = torch.Generator().manual_seed(6)
+    T, k, D, E = 9, 3, 32, 4
+    z = torch.randn(T * k, D, generator=g).to(device)
+    gate = torch.rand(T, k, generator=g).to(device)
+    counter = torch.tensor([5], dtype=torch.int64, device=device)
+    assert torch.equal(ops.gate_reduce(z, gate, counter, 2), ops.gate_reduce(z, gate)) and int(counter) == 7
+    codes = torch.randint(0, 256, (T * k, D), generator=g, dtype=torch.uint8).to(device)
+    scale = (torch.rand(E, 2, generator=g) + 0.1).to(device)
+    sel = torch.randint(0, E, (T, k), generator=g).to(device)
+    assert torch.equal(ops.gate_reduce_codes(codes, scale, sel, gate, counter, 3),
+                       ops.gate_reduce_codes(codes, scale, sel, gate)) and int(counter) == 10
+    assert ops.gate_reduce(z[:0], gate[:0], counter, 1).shape == (0, D) and int(counter) == 11
+    assert ops.gate_reduce_codes(codes[:0], scale, sel[:0], gate[:0], counter, 1).shape == (0, D) and int(counter) == 12
