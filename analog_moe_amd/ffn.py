@@ -37,6 +37,9 @@ class FFNConfig:
     wmax_down: Optional[torch.Tensor] = None      # modified copies (fp32 [E, 1] or [E, N]); None: taken from them
     seed_bump: int = 0                            # added to noise_seed_dev by the forward's last launch (eager calls
                                                   # only: not among the fields the opaque operators take)
+    down_ready: Optional["torch.cuda.Event"] = None  # the down-projection's weights and wmax_down are made on another
+                                                  # stream: the current one waits for this event before it reads them
+                                                  # (eager calls only, as seed_bump)
 
 
 _SIDE_STREAMS = {}
@@ -119,6 +122,8 @@ def ffn_forward(x, keys, values, input_range, gate, sel_idx, cfg: FFNConfig):
                       noise_seed_dev=cfg.noise_seed_dev, xq_ir=ir_dn[:, 0].contiguous() if chain else None,
                       xq_inp_res=cfg.inp_res, **common)
     p1, p1q = p1 if chain else (p1, None)
+    if cfg.down_ready is not None:
+        main.wait_event(cfg.down_ready)
     down = dict(ir=ir_dn, bounds=cfg.bounds_down, noise=cfg.noise_down, noise_seed=cfg.noise_seed + 1, wmax=wd,
                 noise_seed_dev=cfg.noise_seed_dev, x_is_quantized=chain, **common)
     # the gate reduction follows the last launch that draws noise: it moves the device seed word on

@@ -17,6 +17,7 @@ implemented instead of asserted off (:152-160); output noise is drawn inside the
 """
 from __future__ import annotations
 
+import contextlib
 import math
 from functools import partial
 from typing import Callable, Optional, Tuple
@@ -29,7 +30,7 @@ from .config import (AIHWKITTorchInferenceRPUConfig, TorchInferenceRPUConfig, en
 from .cvmm import CVMM, AnalogExt, CVMMSel, cvmm_prepare_sel2, cvmm_std
 from . import library  # noqa: F401  (registers the amoe:: operators)
 from . import ops
-from .ffn import FFNConfig, moe_ffn
+from .ffn import FFNConfig, _side_stream, moe_ffn
 
 
 class MoEConifgError(Exception):
@@ -661,12 +662,31 @@ class AnalogSigmaMoELayer(SigmaMoELayer):
         drew = False
         if (self.training or self.rpu_config.modifier.enable_during_test) and self._modifier_on():
             drew = self.noise_mode != "injected"
-            # the output noise and the ADC keep following the max |W| of the unmodified weights
-            # (moe_layer_aihwkit_lightning.py:458-489)
-            if noisy or cfg.out_bound > 0:
-                cfg.wmax_up = torch.ops.amoe.weight_abs_max(keys.detach(), cfg.noise_per_channel)
-                cfg.wmax_down = torch.ops.amoe.weight_abs_max(values.detach(), cfg.noise_per_channel)
-            keys, values = self._modified(keys, is_down=False), self._modified(values, is_down=True)
+            # The modified copies depend on the parameters only: called eagerly they are made on a second stream, the
+            # up-projection's next to the expert sort and the down-projection's next to the up-projection (which
+            # waits for its own copy only).  The output noise and the ADC keep following the max |W| of the
+            # unmodified weights (moe_layer_aihwkit_lightning.py:458-489)
+            want_wmax = noisy or cfg.out_bound > 0
+            fork = x.is_cuda and not torch.compiler.is_compiling()
+            main = torch.cuda.current_stream() if fork else None
+            side = _side_stream(x.device) if fork else None
+            if fork:
+                side.wait_stream(main)
+            with (torch.cuda.stream(side) if fork else contextlib.nullcontext()):
+                if want_wmax:
+                    cfg.wmax_up = torch.ops.amoe.weight_abs_max(keys.detach(), cfg.noise_per_channel)
+                keys = self._modified(keys, is_down=False)
+                if fork:
+                    main.wait_event(side.record_event())
+                if want_wmax:
+                    cfg.wmax_down = torch.ops.amoe.weight_abs_max(values.detach(), cfg.noise_per_channel)
+                values = self._modified(values, is_down=True)
+                if fork:
+                    cfg.down_ready = side.record_event()
+            if fork:
+                for t in (keys, values, cfg.wmax_up, cfg.wmax_down):
+                    if t is not None:
+                        t.record_stream(main)
         lead = x.shape[:-1]
         if torch.is_autocast_enabled():            # as CVMM.forward does (cvmm.py:716): compute in the autocast type
             dt = torch.get_autocast_dtype("cuda")
