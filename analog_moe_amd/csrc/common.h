@@ -182,7 +182,7 @@ __device__ __forceinline__ Raw raw_pack(const float (&v)[Elem<T>::kChunk]) {
 __device__ __forceinline__ Raw raw_pack_exact_bf16(const float (&v)[8]) {
   Raw r;
 #pragma unroll
-  for (int j = 0; j < 4; j++) r[j] = (as_u32(v[2 * j]) >> 16) | (as_u32(v[2 * j + 1]) & 0xffff0000u);
+  for (int j = 0; j < 4; j++) r[j] = pack_high_halves(as_u32(v[2 * j + 1]), as_u32(v[2 * j]));
   return r;
 }
 // DAC codes as 16-bit elements of T.  Exact only while the type holds the integers: |code| <= 256 in bf16 (the

@@ -84,6 +84,11 @@ __device__ __forceinline__ void buffer_store_b128_nt(BufRsrc r, u32x4 v, uint32_
 // Nothing is scheduled across this point (the compiler otherwise re-orders a software pipeline to save registers).
 __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
+// the high halves of two words as one word: hi's in the upper half, lo's in the lower (one byte permute)
+__device__ __forceinline__ uint32_t pack_high_halves(uint32_t hi, uint32_t lo) {
+  return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+}
+
 // value held by the first active lane, as a scalar
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }

@@ -28,6 +28,7 @@ inline uint32_t buffer_load_b32(BufRsrc r, uint32_t lane_off) {
 inline void buffer_store_b128_nt(BufRsrc r, u32x4 v, uint32_t lane_off) {
   if ((uint64_t)lane_off + 16 <= r.bytes) std::memcpy(const_cast<unsigned char*>(r.base) + lane_off, &v, 16);
 }
+inline uint32_t pack_high_halves(uint32_t hi, uint32_t lo) { return (hi & 0xffff0000u) | (lo >> 16); }
 // scheduling fences mean nothing to a host compiler
 inline void sched_fence() {}
 
