@@ -400,6 +400,10 @@ def main():
                      "frac": achieved / peak, "traffic": traffic,
                      "flops_per_launch": gemm_flops, "avg_launch_ms": kern[dom],
                      **({} if traffic_note is None else {"traffic_note": traffic_note})},
+        # every launch of the step together, against the memory system: recorded HBM bytes per step over the step time
+        **({} if recorded is None or not recorded.get("step_total") else
+           {"step_hbm": {"bytes_per_step": recorded["step_total"], "achieved_GBps": recorded["step_total"] / ms / 1e6,
+                         "peak_GBps": 8000.0, "frac": recorded["step_total"] / ms / 1e6 / 8000.0}}),
         "launch_ms": {n: round(v, 4) for n, v in sorted(kern.items(), key=lambda kv: -kv[1])},
         "gemm_frac_of_peak": {n.split(" ")[0]: round(gemm_flops / (kern[n] * 1e-3) / peak, 4) for n in gemms},
     }

@@ -51,11 +51,16 @@ def load_traffic(config: str):
         rec = json.load(fh)
     if rec.get("source_digest") != source_digest():
         return None, "the kernel sources changed after the recorded counter run"
-    return {role: v["total_bytes"] for role, v in rec["launches"].items()}, None
+    out = {role: v["total_bytes"] for role, v in rec["launches"].items()}
+    out["step_total"] = rec.get("step_total_bytes")
+    return out, None
 
 
 def family(kernel: str):
     """Which of the three GEMM families a kernel name belongs to (None: a companion)."""
+    if "ws256_kernel<" in kernel:                # <T, weights-K-contiguous, ...>: the input gradient reads W that way
+        args = kernel.split("ws256_kernel<", 1)[1].split(">", 1)[0].split(",")
+        return "xgrad" if args[1].strip() == "true" else "fwd"
     if "fwd256_kernel" in kernel:
         return "fwd"
     if "bwdx256_kernel" in kernel:
@@ -68,8 +73,9 @@ def family(kernel: str):
     return None
 
 
-def read_counter(directory: str, counter: str):
-    """Per role: list of counter readings (one per step); and the copy's reading."""
+def read_counter(directory: str, counter: str, others: dict):
+    """Per role: list of counter readings (one per step); and the copy's reading.  others: filled with the summed
+    readings of the launches that are not one of the six (by kernel name)."""
     files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
     if not files:
         sys.exit(f"no *counter_collection.csv under {directory}")
@@ -87,7 +93,10 @@ def read_counter(directory: str, counter: str):
             copy = val if copy is None else max(copy, val)
             continue
         fam = family(name)
-        if fam is None:
+        if fam is None:                            # a companion launch: summed per kernel over the whole run
+            if "amoe::" in name:
+                short = name.split("(")[0].replace("void ", "").replace("amoe::", "")
+                others[short] = others.get(short, 0.0) + val
             continue
         role = ROLES[fam][seen[fam] % 2]
         seen[fam] += 1
@@ -105,8 +114,9 @@ def main():
     ap.add_argument("--config", default="c3")
     ap.add_argument("--skip-first", type=int, default=1, help="steps at the start (warm-up) left out of the average")
     args = ap.parse_args()
-    fetch, fcopy, kernels = read_counter(args.fetch_dir, "FETCH_SIZE")
-    write, wcopy, _ = read_counter(args.write_dir, "WRITE_SIZE")
+    ofetch, owrite = {}, {}
+    fetch, fcopy, kernels = read_counter(args.fetch_dir, "FETCH_SIZE", ofetch)
+    write, wcopy, _ = read_counter(args.write_dir, "WRITE_SIZE", owrite)
     fscale, wscale = COPY_BYTES / (fcopy * 1024.0), COPY_BYTES / (wcopy * 1024.0)
     launches = {}
     print(f"copy of {COPY_BYTES >> 20} MiB reads FETCH_SIZE {fcopy:.0f}, WRITE_SIZE {wcopy:.0f} (KiB): "
@@ -121,7 +131,19 @@ def main():
             launches[role] = {"fetch_size_kib": fk, "write_size_kib": wk, "read_bytes": rb, "write_bytes": wb,
                               "total_bytes": rb + wb, "kernel": kernels[role]}
             print(f"{role:12s} {fk:11.0f} {wk:11.0f} {rb / 1e6:9.1f} {wb / 1e6:9.1f} {(rb + wb) / 1e6:9.1f}  {kernels[role]}")
-    rec = {"workload": args.config, "source_digest": source_digest(),
+    # the other launches of a step, per step (all traced steps: they have no warm-up effects worth a separate average)
+    n_steps = len(fetch["fwd_up"])
+    companions = {}
+    for name in sorted(ofetch, key=lambda n: -(ofetch[n] * fscale + owrite.get(n, 0.0) * wscale)):
+        rb, wb = ofetch[name] * 1024.0 * fscale / n_steps, owrite.get(name, 0.0) * 1024.0 * wscale / n_steps
+        if rb + wb < 1e6:
+            continue
+        companions[name] = {"read_bytes": rb, "write_bytes": wb, "total_bytes": rb + wb}
+        print(f"{name[:40]:40s} {'':>11s} {'':>11s} {rb / 1e6:9.1f} {wb / 1e6:9.1f} {(rb + wb) / 1e6:9.1f}  (per step)")
+    step_total = sum(v["total_bytes"] for v in launches.values()) + sum(v["total_bytes"] for v in companions.values())
+    print(f"all launches of one step: {step_total / 1e6:.0f} MB")
+    rec = {"workload": args.config, "source_digest": source_digest(), "companions": companions,
+           "step_total_bytes": step_total,
            "copy_calibration": {"bytes": COPY_BYTES, "fetch_size_kib": fcopy, "write_size_kib": wcopy,
                                 "fetch_scale": fscale, "write_scale": wscale},
            "launches": launches}
