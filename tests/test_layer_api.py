@@ -306,6 +306,24 @@ def test_library_rejects_bad_arguments_on_the_host():
     assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p, p, 0, 8, p, 2, None) == EINVAL
     assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p, None, 16, 8, p, 2, None) == ENULL
     assert lib.amoe_weight_abs_max_pair(_abi.AMOE_F32, p, 8, 16, p + 2, p, 16, 8, p, 2, None) == EALIGN
+    # the layer's four tables: the weight checks of the pair, then the input-range table's own
+    F32 = _abi.AMOE_F32
+    assert lib.amoe_layer_tables(F32, p, 8, 16, p, p, 16, 8, p, 2, 7, p, 2, 2, p, 1, p, None) == EINVAL      # ir dtype
+    assert lib.amoe_layer_tables(F32, p, 8, 16, p, p, 16, 8, p, 2, F32, p, 2, 3, p, 1, p, None) == EINVAL    # n_up > columns
+    assert lib.amoe_layer_tables(F32, p, 8, 16, p, p, 16, 8, p, 2, F32, p, 2, 2, None, 1, p, None) == ENULL
+    assert lib.amoe_layer_tables(F32, p, 8, 16, p, p, 16, 8, p, 2, F32, p + 2, 2, 2, p, 1, p, None) == EALIGN
+    assert lib.amoe_layer_tables(F32, p, 8, 16, None, p, 16, 8, p, 2, F32, p, 2, 2, p, 1, p, None) == ENULL
+    # per-expert sums: output type, padding columns within the row stride
+    assert lib.amoe_segment_sum(p, p, 2, 1, 5, p, 1, 0, None) == EINVAL                       # output dtype
+    assert lib.amoe_segment_sum(p, p, 2, 1, F32, p, 1, 1, None) == EINVAL                     # padding beyond the row
+    assert lib.amoe_segment_sum(p, p, 2, 1, F32, None, 2, 1, None) == ENULL
+    assert lib.amoe_segment_sum(p, p, 2, 1, F32, p + 2, 2, 1, None) == EALIGN
+    # the counter of the gate reductions is an 8-byte word
+    assert lib.amoe_gate_reduce(F32, p, p, p, 4, 2, 8, p + 4, 1, None) == EALIGN
+    assert lib.amoe_gate_reduce_codes(F32, p, p, p, 1, p, p, 4, 2, 16, p + 4, 1, None) == EALIGN
+    # the codes question answers without launching
+    assert lib.amoe_fwd_codes_supported(None) == 0
+    assert lib.amoe_fwd_codes_supported(fwd()) == 0                                            # fp32, no ADC: values only
     # sum over the heads with the input-range clip
     def ksc(**kw):
         a = _abi.KsumClipArgs(dtype=_abi.AMOE_F32, T=4, k=2, D=32, E=2, full=p, x=p, ldx=32, sel=p, sel_is_i64=1,
