@@ -37,13 +37,15 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
   constexpr int A_ELEMS = kTileRows * LDA, B_ELEMS = BK * LDB;
   constexpr int STAGE = A_ELEMS + B_ELEMS;
   constexpr int LDO = kFCols + 8;                   // staged output rows: 256 columns + 16 bytes
-  constexpr int OUT_ROWS = 64;                      // rows per output pass
-  static_assert(OUT_ROWS * LDO <= 2 * STAGE, "output staging must fit the stage buffers");
+  // the whole 128-row tile is staged at once (all four waves write, one barrier, all threads store): 66 KB, ten more
+  // than the two K-loop stages it overlays, still two workgroups per CU
+  constexpr int OUT_ELEMS = kTileRows * LDO;
+  constexpr int LDS_ELEMS = OUT_ELEMS > 2 * STAGE ? OUT_ELEMS : 2 * STAGE;
   static_assert((!SPLIT2 || ANALOG) && (!NOISE || ANALOG), "the packed first tile holds ADC codes");
   static_assert(!ZCODES || (ANALOG && !SPLIT2), "a result leaves as ADC codes only after a single output quantiser");
   constexpr bool CODES = A_MODE != FA_PLAIN;        // the matrix unit sees integer codes: scale the accumulator
 
-  __shared__ __attribute__((aligned(16))) T sStage[2 * STAGE];
+  __shared__ __attribute__((aligned(16))) T sStage[LDS_ELEMS];
   __shared__ int sOrow[kTileRows];
   __shared__ int sDesc[kMaxDesc][4];
   __shared__ int sWave[4];
@@ -377,43 +379,38 @@ __global__ __launch_bounds__(kThreads, 2) void fwd256_kernel(const RowsParams p)
       const int64_t ldd = pass == 0 ? p.ldo : p.ldxq;
       T* __restrict__ sOut = sStage;
 #pragma unroll
-      for (int h = 0; h < 2; h++) {             // rows 64 h .. 64 h + 63: the waves of row half h
-        if (wr == h) {
+      for (int ti = 0; ti < 2; ti++) {
+        const int rl = wr * 64 + ti * 32 + l32;
 #pragma unroll
-          for (int ti = 0; ti < 2; ti++) {
-            const int rl = ti * 32 + l32;
+        for (int fi = 0; fi < 4; fi++)
 #pragma unroll
-            for (int fi = 0; fi < 4; fi++)
+          for (int q = 0; q < 4; q++) {
+            float v[4];
 #pragma unroll
-              for (int q = 0; q < 4; q++) {
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
-                if (pass == 1) as_codes(v);
-                store4<T>(&sOut[rl * LDO + wc * 128 + fi * 32 + 8 * q + 4 * lh], v, 4, true);
-              }
+            for (int j = 0; j < 4; j++) v[j] = acc[fi][ti][4 * q + j];
+            if (pass == 1) as_codes(v);
+            store4<T>(&sOut[rl * LDO + wc * 128 + fi * 32 + 8 * q + 4 * lh], v, 4, true);
           }
-        }
-        __syncthreads();
-        constexpr int OCPR = kFCols / CH;          // 32 chunks per row
-        constexpr int ORPP = kThreads / OCPR;      // 8 rows per pass of the workgroup
-        constexpr int NROW = 4;                    // rows in flight per thread (the accumulators are still live)
-#pragma unroll
-        for (int i0 = 0; i0 < OUT_ROWS / ORPP; i0 += NROW) {
-          Raw seg[NROW];
-          int orow[NROW];
-#pragma unroll
-          for (int i = 0; i < NROW; i++) {
-            const int rl = tid / OCPR + ORPP * (i0 + i);
-            orow[i] = sOrow[h * OUT_ROWS + rl];
-            seg[i] = *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
-          }
-#pragma unroll
-          for (int i = 0; i < NROW; i++)
-            if (orow[i] >= 0) store_streaming(DST + (int64_t)orow[i] * ldd + c0 + (tid % OCPR) * CH, seg[i]);
-        }
-        __syncthreads();
       }
+      __syncthreads();
+      constexpr int OCPR = kFCols / CH;          // 32 chunks per row
+      constexpr int ORPP = kThreads / OCPR;      // 8 rows per pass of the workgroup
+      constexpr int NROW = 4;                    // rows in flight per thread (the accumulators are still live)
+#pragma unroll
+      for (int i0 = 0; i0 < kTileRows / ORPP; i0 += NROW) {
+        Raw seg[NROW];
+        int orow[NROW];
+#pragma unroll
+        for (int i = 0; i < NROW; i++) {
+          const int rl = tid / OCPR + ORPP * (i0 + i);
+          orow[i] = sOrow[rl];
+          seg[i] = *reinterpret_cast<const Raw*>(&sOut[rl * LDO + (tid % OCPR) * CH]);
+        }
+#pragma unroll
+        for (int i = 0; i < NROW; i++)
+          if (orow[i] >= 0) store_streaming(DST + (int64_t)orow[i] * ldd + c0 + (tid % OCPR) * CH, seg[i]);
+      }
+      __syncthreads();
     };
     emit(std::integral_constant<int, 0>{});
     if (want_xq) emit(std::integral_constant<int, 1>{});
